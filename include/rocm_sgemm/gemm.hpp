@@ -11,8 +11,10 @@
 // All three pointers are device memory owned by the caller, dense and packed in the layout named
 // by the template arguments.  The call enqueues on `stream` and returns without synchronising.
 // Throws std::runtime_error when no kernel exists for the selected config (as the reference does,
-// kernel_launcher.hpp:89-94) and std::invalid_argument for null pointers or zero dimensions (the
-// reference does not validate; it lets the zero-sized launch fail).
+// kernel_launcher.hpp:89-94) and nothing else: like the reference, which does not validate its
+// arguments and leaves a failed launch to the caller's hipPeekAtLastError, a call with a zero
+// dimension or a null pointer returns normally; it enqueues nothing, and rocm_sgemm_last_error()
+// (<rocm_sgemm.h>) says why.  Strict status codes are what the C ABI is for.
 #ifndef ROCM_SGEMM_GEMM_HPP
 #define ROCM_SGEMM_GEMM_HPP
 

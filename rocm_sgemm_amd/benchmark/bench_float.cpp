@@ -57,6 +57,8 @@
 #include <hip/hip_runtime.h>
 #include <rocm_sgemm/gemm.hpp>
 
+#include "sampled_check.hpp"
+
 #ifdef BENCH_WITH_ROCBLAS
 #include <rocblas/rocblas.h>
 #endif
@@ -266,25 +268,12 @@ void print_row(const std::string& name, const timing& t, double bytes, const std
     std::fflush(stdout);
 }
 
-// max |C - C_ref| / (K max|A| max|B|) over 256 sampled entries, C_ref accumulated in fp64
+// max |C - C_ref| / (K max|A| max|B|) over 256 sampled entries, C_ref accumulated in fp64; NaN
+// when a sampled output is NaN (callers test `err <= tolerance`, which NaN fails)
 double sampled_error(const std::vector<float>& C, const std::vector<float>& A, const std::vector<float>& B,
                      size_t M, size_t N, size_t K, bool a_col, bool b_col, bool c_col)
 {
-    float amax = 0, bmax = 0;
-    for(float v : A) amax = std::max(amax, std::fabs(v));
-    for(float v : B) bmax = std::max(bmax, std::fabs(v));
-    std::mt19937_64 gen(12345);
-    double          worst = 0;
-    for(int s = 0; s < 256; ++s)
-    {
-        const size_t i = s < 4 ? (s & 1 ? M - 1 : 0) : gen() % M;
-        const size_t j = s < 4 ? (s & 2 ? N - 1 : 0) : gen() % N;
-        double       acc = 0;
-        for(size_t k = 0; k < K; ++k)
-            acc += static_cast<double>(A[at(a_col, M, K, i, k)]) * B[at(b_col, K, N, k, j)];
-        worst = std::max(worst, std::fabs(C[at(c_col, M, N, i, j)] - acc));
-    }
-    return worst / (static_cast<double>(K) * amax * bmax);
+    return rocm_sgemm::check::sampled_scaled_error(C.data(), A.data(), B.data(), M, N, K, a_col, b_col, c_col);
 }
 
 // The reference's CPU GEMM (test/test.hpp:30-45): i-j-k, fp32 accumulator; rows dealt to threads.

@@ -85,10 +85,18 @@ bool aligned16(const void* p)
 // allocation at all once the buffer is large enough.  (A stream-ordered hipMallocAsync /
 // hipFreeAsync pair per call was measured to stall the host until the GPU had caught up, which
 // serialises back-to-back calls.)  Calls on different streams get different buffers, so they may
-// overlap; the table itself is guarded by a mutex.
-// While a stream is being captured into a graph no memory can be allocated synchronously: a
-// buffer that is already large enough is used as it is, otherwise the call falls back to a
-// stream-ordered allocation, which the capture records as allocation / free nodes.
+// overlap.
+// Locking: the table is guarded by one mutex that is held for the lookup only; every buffer has a
+// mutex of its own that a call holds from "got the pointer" until it has enqueued everything that
+// uses the buffer.  Growing a buffer frees the old one after waiting for the device, which is only
+// safe if no other thread is between those two points on the same buffer; threads on different
+// streams never wait for each other.  Table nodes are never erased (release_workspaces() empties
+// them in place), so a pointer to a node stays valid for the life of the process.
+// A stream that is being captured into a graph NEVER gets the library's buffer: its address would
+// be baked into the graph's kernel nodes, and a later growth or release_workspaces() would leave
+// every replay reading and writing freed memory.  A captured call always takes a stream-ordered
+// allocation instead, which the capture records as allocation / free nodes: the graph owns its
+// workspace.
 // hipStreamPerThread is one handle value that names a different stream in every host thread, so
 // for it the calling thread is part of the key (0 for every other stream).
 struct workspace_key
@@ -105,58 +113,63 @@ struct workspace_key
 };
 struct workspace_buffer
 {
-    void*  ptr   = nullptr;
-    size_t bytes = 0;
+    std::mutex in_use; // held by a call from taking `ptr` until its kernels are enqueued
+    void*      ptr   = nullptr;
+    size_t     bytes = 0;
 };
-std::mutex                                    workspace_lock;
-std::map<workspace_key, workspace_buffer>     workspaces;
+std::mutex                                workspace_table_lock;
+std::map<workspace_key, workspace_buffer> workspaces;
 
 // Returns the buffer in *ptr; *stream_ordered is set when the caller must hipFreeAsync it.
-// `guard` comes back locked and must stay so until the caller has enqueued everything that uses
-// the buffer: growing a buffer frees the old one after waiting for the device, which is only
-// safe if no other thread is between "got the pointer" and "enqueued the kernels".
+// Otherwise `guard` comes back holding the buffer's mutex and must stay so until the caller has
+// enqueued everything that uses the buffer.
 hipError_t workspace_get(void** ptr, size_t bytes, hipStream_t stream, bool* stream_ordered,
                          std::unique_lock<std::mutex>& guard)
 {
     *stream_ordered = false;
-    int device      = 0;
-    hipError_t err  = hipGetDevice(&device);
-    if(err != hipSuccess) return err;
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if(hipStreamIsCapturing(stream, &capture) != hipSuccess)
     {
         (void)hipGetLastError();
         capture = hipStreamCaptureStatusNone;
     }
-    guard = std::unique_lock<std::mutex>(workspace_lock);
-    const size_t thread = stream == hipStreamPerThread ? std::hash<std::thread::id>{}(std::this_thread::get_id()) : 0;
-    workspace_buffer& buf = workspaces[workspace_key{device, stream, thread}];
-    if(buf.bytes >= bytes)
-    {
-        *ptr = buf.ptr;
-        return hipSuccess;
-    }
     if(capture != hipStreamCaptureStatusNone)
     {
         *stream_ordered = true;
         return hipMallocAsync(ptr, bytes, stream);
     }
+    int        device = 0;
+    hipError_t err    = hipGetDevice(&device);
+    if(err != hipSuccess) return err;
+    const size_t thread = stream == hipStreamPerThread ? std::hash<std::thread::id>{}(std::this_thread::get_id()) : 0;
+    workspace_buffer* buf;
+    {
+        std::lock_guard<std::mutex> table(workspace_table_lock);
+        buf = &workspaces[workspace_key{device, stream, thread}];
+    }
+    guard = std::unique_lock<std::mutex>(buf->in_use);
+    if(buf->bytes >= bytes)
+    {
+        *ptr = buf->ptr;
+        return hipSuccess;
+    }
     // Grow.  The old buffer may still be in use by work queued on this stream; hipFree waits for
     // the device, which is acceptable for an event that happens a handful of times per process.
-    if(buf.ptr != nullptr)
+    if(buf->ptr != nullptr)
     {
-        (void)hipFree(buf.ptr);
-        buf = workspace_buffer{};
+        (void)hipFree(buf->ptr);
+        buf->ptr   = nullptr;
+        buf->bytes = 0;
     }
     const size_t want = bytes + bytes / 4; // head room: slightly larger problems do not regrow
-    err               = hipMalloc(&buf.ptr, want);
+    err               = hipMalloc(&buf->ptr, want);
     if(err != hipSuccess)
     {
-        buf = workspace_buffer{};
+        buf->ptr = nullptr;
         return err;
     }
-    buf.bytes = want;
-    *ptr      = buf.ptr;
+    buf->bytes = want;
+    *ptr       = buf->ptr;
     return hipSuccess;
 }
 
@@ -180,7 +193,7 @@ int compute_units()
 
 void release_workspaces()
 {
-    std::lock_guard<std::mutex> guard(workspace_lock);
+    std::lock_guard<std::mutex> table(workspace_table_lock);
     int                         current = -1;
     if(hipGetDevice(&current) != hipSuccess)
     {
@@ -189,13 +202,15 @@ void release_workspaces()
     }
     for(auto& kv : workspaces)
     {
+        std::lock_guard<std::mutex> in_use(kv.second.in_use); // no call is about to enqueue on it
         if(kv.second.ptr != nullptr)
         {
             (void)hipSetDevice(kv.first.device);
             (void)hipFree(kv.second.ptr); // waits for the device: nothing can still be using it
+            kv.second.ptr   = nullptr;
+            kv.second.bytes = 0;
         }
     }
-    workspaces.clear();
     if(current >= 0) (void)hipSetDevice(current); // the caller's current device is left as it was
 }
 

@@ -10,7 +10,6 @@
 #include <cstdio>
 #include <cstdlib>
 #include <random>
-#include <stdexcept>
 #include <vector>
 
 #include <rocm_sgemm/gemm.hpp>
@@ -93,19 +92,15 @@ int main()
     ok &= run_case<c, r, c>(320, 512, 512, stream);
     ok &= run_case<c, c, r>(320, 512, 512, stream);
     ok &= run_case<c, c, c>(320, 512, 512, stream);
-    // zero-sized problem: the library reports it as an exception (the reference lets the launch fail)
-    bool threw = false;
-    try
+    // zero-sized problem, no try block: like the reference the entry point does not throw for its
+    // arguments; nothing is enqueued and the stream stays usable
     {
         float* p = reinterpret_cast<float*>(0x1000);
         rocm_sgemm::gemm<rocm_sgemm::m_layout::row_major, rocm_sgemm::m_layout::row_major,
                          rocm_sgemm::m_layout::row_major>(p, p, p, 0, 4, 4, stream);
+        HIP_OK(hipStreamSynchronize(stream));
+        std::printf("zero dimension -> returns without launching: PASS\n");
     }
-    catch(const std::invalid_argument&)
-    {
-        threw = true;
-    }
-    std::printf("zero dimension -> std::invalid_argument: %s\n", threw ? "PASS" : "FAIL");
     HIP_OK(hipStreamDestroy(stream));
-    return ok && threw ? 0 : 1;
+    return ok ? 0 : 1;
 }

@@ -449,6 +449,25 @@ def test_nothing_outside_an_operand_reaches_the_result(la, lb, lc):
             assert bad.size == 0, (cfg, M, N, K, off, bad[:5], got[bad[:5]], want[bad[:5]])
 
 
+def test_sixteen_byte_loads_that_straddle_the_end_of_a_padded_operand():
+    """16-byte direct-to-LDS loads are chosen when pointers and leading dimensions are 16-byte
+    aligned and K is a multiple of 4 - also when a row-contiguous operand's own width is not a
+    multiple of 4 under a padded leading dimension (column-major A with M = 130, lda = 132).  The
+    last 16-byte piece of the final depth line then straddles the operand's end: its first two
+    floats are data, the other two lie beyond the allocation.  The range check must drop the
+    out-of-range dwords only, not the whole piece.  Padding holds NaN, the buffers end exactly at
+    the operands' extents, integer-valued data: bit-exact or wrong."""
+    rng = np.random.default_rng(61)
+    for fam in [f for f in rs.family() if f.stages > 0]:
+        cfg = dict(fam.as_dict(), split_k=1, group_m=2, wave_slots=1)
+        for (M, N, K, la, lb, lc, pads) in [(130, 64, 72, 1, 0, 0, (2, 0, 0)),   # X row-contiguous, ragged
+                                            (64, 134, 72, 0, 0, 0, (0, 2, 0)),   # Y column-contiguous, ragged
+                                            (130, 134, 40, 1, 0, 0, (2, 2, 0)),  # both
+                                            (130, 134, 40, 1, 0, 1, (2, 2, 2))]:  # swapped for a column-major C
+            _announce("straddling_piece", cfg, M, N, K, la, lb, lc, pads)
+            check_strided_batched_exact(rng, M, N, K, la, lb, lc, 1, 1, 0, pads, config=cfg)
+
+
 def test_stream_k_tail_matches_plain_run_and_is_deterministic():
     """The stream-K tail (K range of a short last wave of tiles dealt out to all slots) changes
     only the summation order of the affected tiles: results stay within the fp64 tolerance, repeat
@@ -563,6 +582,54 @@ def test_call_can_be_captured_in_a_hip_graph_and_replayed():
         rs.gemm_with_config(cfg, eager, dA, dB, M, N, K, stream=torch.cuda.current_stream())
         torch.cuda.synchronize()
         assert torch.equal(replayed, eager), seed
+
+
+@pytest.mark.parametrize("what", ["split_k", "stream_k_tail"])
+def test_captured_call_with_partials_owns_its_workspace(what):
+    """A call that needs a workspace (split-K, stream-K tail) recorded into a HIP graph must not
+    bake the library's per-stream buffer into the graph: that buffer is freed when a later eager
+    call on the stream outgrows it and by release_workspaces().  The order below is the usual one
+    (eager warm-up creates the buffer, capture follows, a bigger product comes later); every
+    replay, with fresh integer-valued inputs, must equal the int64 product bit for bit."""
+    import torch
+    rng = np.random.default_rng(77)
+    M, N, K = 300, 260, 1000
+    base = rs.family()[0].as_dict()
+    cfg = dict(base, split_k=4, wave_slots=1) if what == "split_k" else dict(base, split_k=1, wave_slots=3)
+    _announce("graph_capture_workspace", what, cfg, M, N, K)
+    A, B, C = int_matrices(rng, M, N, K)
+    dA, dB = to_device(A.reshape(-1)), to_device(B.reshape(-1))
+    dC = torch.zeros(M * N, dtype=torch.float32, device="cuda:0")
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        rs.gemm_with_config(cfg, dC, dA, dB, M, N, K, stream=stream)  # the stream now has a buffer
+    stream.synchronize()
+    assert np.array_equal(dC.cpu().numpy().reshape(M, N), C)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        rs.gemm_with_config(cfg, dC, dA, dB, M, N, K, stream=torch.cuda.current_stream())
+    # a larger eager product on the same stream outgrows the stream's buffer; then everything the
+    # library holds is given back
+    M2, N2, K2 = 700, 650, 1200
+    A2, B2, C2 = int_matrices(rng, M2, N2, K2)
+    dC2 = torch.zeros(M2 * N2, dtype=torch.float32, device="cuda:0")
+    rs.gemm_with_config(dict(base, split_k=6, wave_slots=1), dC2, to_device(A2.reshape(-1)),
+                        to_device(B2.reshape(-1)), M2, N2, K2, stream=stream)
+    stream.synchronize()
+    assert np.array_equal(dC2.cpu().numpy().reshape(M2, N2), C2)
+    rs.release_workspaces()
+    filler = torch.full((64 << 20,), float("nan"), device="cuda:0")  # reuse whatever was freed
+    for _ in range(3):
+        A, B, C = int_matrices(rng, M, N, K)
+        dA.copy_(to_device(A.reshape(-1)))
+        dB.copy_(to_device(B.reshape(-1)))
+        dC.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(dC.cpu().numpy().reshape(M, N), C)
+    del filler
 
 
 # ---- general form: leading dimensions, strided batches, alpha / beta ---------------------------------

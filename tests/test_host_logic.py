@@ -514,3 +514,54 @@ def test_report_parses_bench_rows_and_builds_the_table(tmp_path):
     out = tmp_path / "r.md"
     assert report.main(["--log", str(log), "--output", str(out)]) == 0
     assert "rocBLAS (best C)" in out.read_text() and "hipBLASLt (best C)" in out.read_text()
+
+
+# ---- sampled correctness gate of the tuner trial binary and bench_float --------------------------
+
+SAMPLED_CHECK_PROBE = r"""
+#include <cstdio>
+#include <limits>
+#include <vector>
+#include "sampled_check.hpp"
+int main()
+{
+    using namespace rocm_sgemm::check;
+    const size_t M = 37, N = 29, K = 53;
+    std::vector<float> A(M * K), B(K * N), C(M * N);
+    for(size_t i = 0; i < A.size(); ++i) A[i] = static_cast<float>((i * 7 + 3) % 11) - 5.0f;
+    for(size_t i = 0; i < B.size(); ++i) B[i] = static_cast<float>((i * 5 + 1) % 9) - 4.0f;
+    for(size_t i = 0; i < M; ++i)
+        for(size_t j = 0; j < N; ++j)
+        {
+            float acc = 0.0f;
+            for(size_t k = 0; k < K; ++k) acc += A[i * K + k] * B[k * N + j];
+            C[i * N + j] = acc;
+        }
+    const double good = sampled_scaled_error(C.data(), A.data(), B.data(), M, N, K, false, false, false);
+    // every entry sampled (samples >> M * N), one NaN anywhere must be seen
+    std::vector<float> one_nan = C;
+    one_nan[5 * N + 7]         = std::numeric_limits<float>::quiet_NaN();
+    const double nan_err = sampled_scaled_error(one_nan.data(), A.data(), B.data(), M, N, K, false, false, false, 20000);
+    std::vector<float> unwritten(M * N, std::numeric_limits<float>::quiet_NaN());
+    const double all_nan = sampled_scaled_error(unwritten.data(), A.data(), B.data(), M, N, K, false, false, false);
+    std::vector<float> off = C;
+    off[0] += 1.0f; // corner (0, 0) is always sampled
+    const double wrong = sampled_scaled_error(off.data(), A.data(), B.data(), M, N, K, false, false, false);
+    std::printf("%d %d %d %d\n", within_tolerance(good), within_tolerance(nan_err), within_tolerance(all_nan),
+                within_tolerance(wrong));
+    return 0;
+}
+"""
+
+
+def test_sampled_check_fails_on_nan_and_unwritten_outputs(tmp_path):
+    """The gate behind `ok 0|1` of a tuner trial and behind bench_float --verify: an exact product
+    passes; a NaN sample, an output left at its NaN pre-fill and a wrong value all fail
+    (std::max(worst, NaN) would have returned `worst` and passed them)."""
+    src = tmp_path / "probe.cpp"
+    src.write_text(SAMPLED_CHECK_PROBE)
+    exe = tmp_path / "probe"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-I", os.path.join(REPO, "rocm_sgemm_amd", "benchmark"),
+                    str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert out == ["1", "0", "0", "0"], out
