@@ -53,15 +53,34 @@ def tflops(m, n, k, ms):
     return 2.0 * m * n * k / (ms * 1e-3) * 1e-12
 
 
-def timed_launches(fn, steps, warmup):
-    """Per-launch event-pair timings (ms) of `steps` launches after `warmup`, plus the wall time
-    (ms) of the timed region bracketed by device synchronisation."""
+WARMUP_MIN_MS = 40.0  # sustained launches before any timed region (the clocks need tens of ms)
+
+
+def timed_launches(fn, steps, warmup, min_warm_ms=WARMUP_MIN_MS):
+    """The one timing protocol of this file.  Warm-up: at least `warmup` launches AND at least
+    `min_warm_ms` of sustained launches (after an idle gap the GPU needs tens of milliseconds of
+    work to reach its full clock, whatever the launch count).  Then `steps` launches queued back to
+    back, each bracketed by an event pair on the launch stream, closed by ONE synchronisation.
+    Returns the per-launch durations (ms), the wall time (ms) of the timed region, and the device
+    time (ms) from the first launch's start event to the last one's stop event - the sustained
+    rate, which unlike the per-launch figures includes launch gaps."""
     import torch
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]  # before the warm-up:
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]   # no idle gap after it
+    warmed_ms, launched, batch = 0.0, 0, 5
+    w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    while launched < warmup or warmed_ms < min_warm_ms:
+        w0.record()
+        for _ in range(batch):
+            fn()
+        w1.record()
+        w1.synchronize()
+        took = max(w0.elapsed_time(w1), 1e-3)
+        warmed_ms += took
+        launched += batch
+        # next batch: what is left of the warm-up time at the rate just seen
+        left = max(min_warm_ms - warmed_ms, 0.0) * batch / took
+        batch = int(max(warmup - launched, min(left, 5000), 1))
     t0 = time.perf_counter()
     for i in range(steps):
         starts[i].record()
@@ -69,7 +88,16 @@ def timed_launches(fn, steps, warmup):
         stops[i].record()
     torch.cuda.synchronize()  # one synchronisation for the whole timed region
     wall_ms = (time.perf_counter() - t0) * 1e3
-    return [s.elapsed_time(e) for s, e in zip(starts, stops)], wall_ms
+    return [s.elapsed_time(e) for s, e in zip(starts, stops)], wall_ms, starts[0].elapsed_time(stops[-1])
+
+
+def summary(m, n, k, ms, span_ms):
+    avg = sum(ms) / len(ms)
+    return {"avg_tflops": round(tflops(m, n, k, avg), 2),
+            "min_time_tflops": round(tflops(m, n, k, min(ms)), 2),
+            "pct_peak_avg": round(100 * tflops(m, n, k, avg) / PEAK_TFLOPS, 1),
+            "avg_ms": round(avg, 5),
+            "sustained_tflops": round(tflops(m, n, k, span_ms / len(ms)), 2)}
 
 
 def uniform_device(count, seed):
@@ -80,6 +108,8 @@ def uniform_device(count, seed):
 
 
 def bench_layouts(rs, sizes, steps, warmup):
+    """The reference bench's default shapes (reference benchmark/gemm/bench.cpp:240-303,
+    docs/square.md:9-24): cubes x the four A/B storage orders x both C orders, uniform inputs."""
     import torch
     out = {}
     names = {0: "row", 1: "col"}
@@ -93,12 +123,9 @@ def bench_layouts(rs, sizes, steps, warmup):
                 for lb in (0, 1):
                     def fn():
                         rs.gemm(dC, dA, dB, size, size, size, lc, la, lb, stream=stream)
-                    ms, _ = timed_launches(fn, n_steps, warmup)
+                    ms, _, span = timed_launches(fn, n_steps, warmup)
                     key = f"{size}^3 A={names[la]} B={names[lb]} C={names[lc]}"
-                    avg = sum(ms) / len(ms)
-                    out[key] = {"avg_tflops": round(tflops(size, size, size, avg), 2),
-                                "min_time_tflops": round(tflops(size, size, size, min(ms)), 2),
-                                "pct_peak_avg": round(100 * tflops(size, size, size, avg) / PEAK_TFLOPS, 1)}
+                    out[key] = summary(size, size, size, ms, span)
         del dA, dB, dC
     return out
 
@@ -109,7 +136,7 @@ RECT_SHAPES = [(8192, 8192, 1024), (1024, 1024, 16384), (128, 4096, 4096), (4096
 
 def bench_shapes(rs, steps, warmup):
     """The rectangular, unaligned and large row-major configurations, with the vendor library
-    (torch.matmul) timed on the same operands for context."""
+    (torch.matmul) timed on the same operands, by the same protocol, for context."""
     import torch
     torch.backends.cuda.matmul.allow_tf32 = False
     out = {}
@@ -119,17 +146,14 @@ def bench_shapes(rs, steps, warmup):
         dC = torch.empty(m * n, dtype=torch.float32, device="cuda:0")
         flop_ms = 2.0 * m * n * k / 140e9  # rough duration, to keep every shape to a fraction of a second
         n_steps = max(5, min(steps, int(200 / max(flop_ms, 0.01))))
-        ms, _ = timed_launches(lambda: rs.gemm(dC, dA, dB, m, n, k, stream=stream), n_steps,
-                               max(warmup, min(50, int(40 / max(flop_ms, 0.01)))))
-        avg = sum(ms) / len(ms)
+        ms, _, span = timed_launches(lambda: rs.gemm(dC, dA, dB, m, n, k, stream=stream), n_steps, warmup)
         a2, b2 = dA.view(m, k), dB.view(k, n)
-        vms, _ = timed_launches(lambda: torch.matmul(a2, b2), n_steps,
-                                max(warmup, min(50, int(40 / max(flop_ms, 0.01)))))
-        vavg = sum(vms) / len(vms)
-        out[f"{m}x{n}x{k}"] = {"avg_tflops": round(tflops(m, n, k, avg), 2),
-                               "min_time_tflops": round(tflops(m, n, k, min(ms)), 2),
-                               "avg_ms": round(avg, 4),
-                               "vendor_avg_tflops": round(tflops(m, n, k, vavg), 2)}
+        vms, _, vspan = timed_launches(lambda: torch.matmul(a2, b2), n_steps, warmup)
+        row = summary(m, n, k, ms, span)
+        row["vendor_avg_tflops"] = round(tflops(m, n, k, sum(vms) / len(vms)), 2)
+        row["vendor_sustained_tflops"] = round(tflops(m, n, k, vspan / len(vms)), 2)
+        row["kernel_config"] = rs.find_config(m, n, k).as_dict()
+        out[f"{m}x{n}x{k}"] = row
         del dA, dB, dC, a2, b2
     return out
 
@@ -143,16 +167,18 @@ def bench_context(sizes, steps, warmup):
         a = uniform_device(size * size, 3).view(size, size)
         b = uniform_device(size * size, 4).view(size, size)
         n_steps = steps if size <= 4096 else max(10, steps // 5)
-        ms, _ = timed_launches(lambda: torch.matmul(a, b), n_steps, warmup)
-        avg = sum(ms) / len(ms)
-        out[f"torch.matmul fp32 {size}^3 (hipBLASLt/rocBLAS)"] = {
-            "avg_tflops": round(tflops(size, size, size, avg), 2),
-            "min_time_tflops": round(tflops(size, size, size, min(ms)), 2)}
+        ms, _, span = timed_launches(lambda: torch.matmul(a, b), n_steps, warmup)
+        out[f"torch.matmul fp32 {size}^3 (hipBLASLt/rocBLAS)"] = summary(size, size, size, ms, span)
     return out
 
 
-def cpu_baseline():
-    """The reference CPU GEMM on this host: single thread, i-j-k, fp32 accumulator, 1024^3.
+def cpu_baseline(max_seconds=12.0):
+    """The reference CPU GEMM on this host (reference test/test.hpp:30-45: i-j-k, fp32
+    accumulator): one thread at 1024^3, as the reference runs it; the same loop nest with the rows
+    of C dealt out to threads at 1024^3; and the all-threads leg at 4096^3 on a bounded sample -
+    the first R rows of C against the whole of B, which keeps the real access pattern (a
+    column-strided walk over a 64 MiB B), with R sized to about `max_seconds` and the figure for
+    all 4096 rows extrapolated by row count and labelled so.
     This leg is the only place where the benchmark touches the oracle (as a baseline, never as the
     thing measured): the CPU restatement, and - where it has been built - the reference's own GPU
     kernel timed on this GPU at 4096^3 row-major for context."""
@@ -162,7 +188,13 @@ def cpu_baseline():
     t0 = time.perf_counter()
     oracle.sgemm_f32(a, b, n, n, n, 0, 0, 0, threads=1)
     one = time.perf_counter() - t0
-    cores = min(16, os.cpu_count() or 1)
+    host_cores = os.cpu_count() or 1
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = host_cores
+    # threads actually used: what this process may run on, at most the 16 a one-GPU box grants
+    cores = max(1, min(usable, 16))
     t0 = time.perf_counter()
     oracle.sgemm_f32(a, b, n, n, n, 0, 0, 0, threads=cores)
     many = time.perf_counter() - t0
@@ -171,9 +203,30 @@ def cpu_baseline():
            "sample": "one 1024^3 row-major SGEMM, uniform[-1,1) seed 0, reference loop nest "
                      "(i-j-k, fp32 accumulator), 1 thread as the reference runs it",
            "seconds": round(one, 3),
+           "host_cores": host_cores, "usable_cores": usable,
            "all_cores": {"value": round(flops / many * 1e-12, 6), "cores": cores,
                          "seconds": round(many, 3),
-                         "note": "same loop nest, rows of C dealt out to threads"}}
+                         "note": "same loop nest at 1024^3, rows of C dealt out to threads"}}
+    # 4096^3 on all threads, bounded
+    big = 4096
+    a4, b4 = oracle.fill_uniform_pair(big, big, big, 0, 0, seed=0)
+    rows = cores  # one row of C per thread first, to size the sample
+    t0 = time.perf_counter()
+    oracle.sgemm_f32(a4[:rows * big], b4, rows, big, big, 0, 0, 0, threads=cores)
+    probe = time.perf_counter() - t0
+    rows = int(min(big, max(cores, cores * int(max_seconds / max(probe, 1e-3)))))
+    t0 = time.perf_counter()
+    oracle.sgemm_f32(a4[:rows * big], b4, rows, big, big, 0, 0, 0, threads=cores)
+    took = time.perf_counter() - t0
+    out["all_cores_4096"] = {
+        "value": round(2.0 * rows * big * big / took * 1e-12, 6), "unit": "TFLOP/s", "cores": cores,
+        "rows_timed": rows, "seconds": round(took, 3),
+        "seconds_for_4096_rows": round(took * big / rows, 1),
+        "extrapolated": rows < big,
+        "note": ("the whole 4096^3 product" if rows == big else
+                 f"first {rows} of 4096 rows of C against the whole of B (the full access pattern); "
+                 "seconds_for_4096_rows is extrapolated by row count")}
+    del a4, b4
     ref = oracle.ref_kernel()
     if ref is not None:
         import torch
@@ -184,18 +237,17 @@ def cpu_baseline():
         def fn():
             ref.ref_kernel_sgemm(0, 0, 0, dC.data_ptr(), dA.data_ptr(), dB.data_ptr(), M, N, K,
                                  stream.cuda_stream)
-        ms, _ = timed_launches(fn, 30, 10)
-        avg = sum(ms) / len(ms)
-        out["reference_gpu_kernel_same_gpu"] = {
-            "avg_tflops": round(tflops(M, N, K, avg), 2),
-            "min_time_tflops": round(tflops(M, N, K, min(ms)), 2),
-            "note": "the reference's kernel_gemm with its own tuned 4096^3 row-major parameters, "
-                    "compiled for gfx950 from the reference sources (context, not a target)"}
+        ms, _, span = timed_launches(fn, 30, 10)
+        out["reference_gpu_kernel_same_gpu"] = dict(
+            summary(M, N, K, ms, span),
+            note="the reference's kernel_gemm with its own tuned 4096^3 row-major parameters, "
+                 "compiled for gfx950 from the reference sources (context, not a target)")
     return out
 
 
 def read_traffic():
-    """HBM bytes per launch from the committed counter summary, or None."""
+    """HBM bytes per launch from the committed counter summary (written by an earlier
+    `bench.py --counters` run of this same workload), or None."""
     try:
         with open(COUNTER_SUMMARY) as f:
             for line in f:
@@ -363,7 +415,7 @@ def main():
     def step():
         rs.gemm(dC, dA, dB, M, N, K, stream=stream)
 
-    times, wall_ms = timed_launches(step, args.steps, args.warmup)
+    times, wall_ms, _ = timed_launches(step, args.steps, args.warmup)
     if not torch.equal(dC.view(torch.int32), dA.view(torch.int32)):
         sys.exit("bench.py: identity-B result differs from A - refusing to report a number")
     avg_ms = sum(times) / len(times)
@@ -371,13 +423,18 @@ def main():
     ms_per_step = wall_ms / args.steps
     cfg = rs.find_config(M, N, K).as_dict()
 
-    traffic = None
     counters = None
     if args.counters:
         counters = counters_report(args.steps, args.warmup)
         write_counter_summary(counters, avg_ms)
         counters.pop("raw", None)
-    traffic = read_traffic()
+        traffic = counters.get("hbm_bytes_per_launch")
+        traffic_source = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes of this run"
+    else:
+        traffic = read_traffic()
+        traffic_source = (None if traffic is None else
+                          "profiles/sgemm_mfma_4096_rrr_counters.txt: rocprofv3 --pmc passes of an "
+                          "earlier `bench.py --counters` run of this workload, not measured in this run")
 
     line = {
         "metric": "SGEMM TFLOPS (avg & min) at 4096^3; % of MI355X FP32 MFMA peak",
@@ -403,12 +460,13 @@ def main():
                                   "min_time": round(100 * tflops(M, N, K, min_ms) / PEAK_TFLOPS, 1)},
         "roofline": {"bound": "mfma", "achieved": round(tflops(M, N, K, avg_ms), 2),
                      "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops(M, N, K, avg_ms) / PEAK_TFLOPS, 4), "traffic": traffic},
+                     "frac": round(tflops(M, N, K, avg_ms) / PEAK_TFLOPS, 4), "traffic": traffic,
+                     "traffic_source": traffic_source},
     }
     if counters is not None:
         line["counters"] = counters
     if not args.no_layouts:
-        line["layouts"] = bench_layouts(rs, (4096, 8192), args.steps, args.warmup)
+        line["layouts"] = bench_layouts(rs, (1024, 2048, 4096, 8192), args.steps, args.warmup)
         line["shapes_row_major"] = bench_shapes(rs, args.steps, args.warmup)
     if not args.no_context:
         line["context"] = bench_context((4096, 8192), args.steps, args.warmup)

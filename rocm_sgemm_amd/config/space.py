@@ -10,8 +10,9 @@ describe a wave32 VALU kernel (thread tiles, threads_n); an MFMA kernel is descr
     waves_m x waves_n   wave64 grid of the workgroup
     mfma                32 -> v_mfma_f32_32x32x2_f32, 16 -> v_mfma_f32_16x16x4_f32
     stages              0 -> operands staged through registers into two LDS stages;
-                        n >= 2 -> loaded straight into a ring of n LDS stages (full tiles only:
-                        problems with ragged edges run the register-staged kernel of the shape)
+                        n >= 2 -> loaded straight into a ring of n LDS stages (ragged problems
+                        run the edge-masked variants of the same kernel: 16-byte loads when the
+                        operand lines are 16-byte aligned, 4-byte loads otherwise)
     split_k, group_m    launch-time only: K slices and tile-order band height
     wave_slots          launch-time only: 0 = deal the K range of a short last wave of tiles out
                         to all CUs (stream-K tail; slots asked from the runtime), 1 = never
@@ -96,7 +97,7 @@ def shape_ok(shape):
         return False
     if (macro_m * k_tile // 4) % threads or (macro_n * k_tile // 4) % threads:
         return False
-    # the edge-masked kernel of a shape is always the register-staged one: both must fit
+    # the register-staged twin of a direct-to-LDS shape is compiled alongside it: both must fit
     if max(max_lds_bytes(macro_m, macro_n, k_tile, 0),
            max_lds_bytes(macro_m, macro_n, k_tile, stages)) > LDS_BYTES_PER_CU:
         return False
