@@ -39,8 +39,13 @@ enum
                                             the condition under which the reference throws
                                             std::runtime_error (kernel_launcher.hpp:89-94) */
     ROCM_SGEMM_STATUS_LAUNCH_FAILED = 3, /* HIP refused the launch or the workspace allocation */
-    ROCM_SGEMM_STATUS_BAD_CONFIG    = 4  /* config fields out of range */
+    ROCM_SGEMM_STATUS_BAD_CONFIG    = 4, /* config fields out of range */
+    ROCM_SGEMM_STATUS_WORKSPACE_TOO_LARGE = 5 /* rocm_sgemm_f32_no_alloc only: the problem's
+                                                 partial products do not fit the fixed scratch */
 };
+
+/* Size of the fixed device scratch array behind rocm_sgemm_f32_no_alloc, per GPU. */
+#define ROCM_SGEMM_NO_ALLOC_SCRATCH_BYTES (128u * 1024u * 1024u)
 
 /*
  * Tuned launch parameters of one table entry.  Takes the place of the reference's 9-int tuple
@@ -94,6 +99,33 @@ int rocm_sgemm_f32(int          layout_c,
                    size_t       N,
                    size_t       K,
                    void*        stream);
+
+/*
+ * The same product as rocm_sgemm_f32 - same config, same kernels, same bits - for callers that
+ * cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  It has no counterpart in the reference (whose kernels never need a
+ * workspace).  rocm_sgemm_f32 keeps the partial products of a split-K or stream-K-tail config in
+ * a workspace it allocates; this entry point keeps them in a fixed array of
+ * ROCM_SGEMM_NO_ALLOC_SCRATCH_BYTES of device memory that is part of the library's code object
+ * (every GPU the library runs on holds it until the process ends) and calls no hipMalloc, hipFree
+ * or other allocating routine.  A problem whose partial products need more than that is refused
+ * with ROCM_SGEMM_STATUS_WORKSPACE_TOO_LARGE and nothing is enqueued (a product of any size whose
+ * config neither splits K nor deals out a tail needs no scratch and always runs).
+ * All calls on one GPU share the array: two calls may not overlap in time on one GPU (calls on
+ * one stream never do; calls on different streams, or replays of graphs that recorded such
+ * calls, must be ordered by the caller).  Nothing in the array needs clearing between calls:
+ * every partial product a call reads it has written itself.
+ */
+int rocm_sgemm_f32_no_alloc(int          layout_c,
+                            int          layout_a,
+                            int          layout_b,
+                            float*       C,
+                            const float* A,
+                            const float* B,
+                            size_t       M,
+                            size_t       N,
+                            size_t       K,
+                            void*        stream);
 
 /*
  * Same product with an explicit config instead of the table lookup.  Replaces the tuner's

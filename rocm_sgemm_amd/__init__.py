@@ -15,7 +15,7 @@ import os
 
 __all__ = [
     "ROW_MAJOR", "COL_MAJOR", "Config", "SgemmError", "NoKernelError", "lib", "lib_path", "gemm",
-    "gemm_with_config", "gemm_strided_batched", "find_config", "nearest_config", "predict_us", "table", "family", "config_supported", "map_workgroup",
+    "gemm_no_alloc", "gemm_with_config", "gemm_strided_batched", "find_config", "nearest_config", "predict_us", "table", "family", "config_supported", "map_workgroup",
     "release_workspaces", "version", "CXX_SYMBOLS", "C_SYMBOLS",
 ]
 
@@ -24,11 +24,13 @@ COL_MAJOR = 1
 _LAYOUT_NAMES = {"row_major": ROW_MAJOR, "col_major": COL_MAJOR, "r": ROW_MAJOR, "c": COL_MAJOR,
                  ROW_MAJOR: ROW_MAJOR, COL_MAJOR: COL_MAJOR}
 
-STATUS_OK, STATUS_INVALID_ARG, STATUS_NO_KERNEL, STATUS_LAUNCH_FAILED, STATUS_BAD_CONFIG = range(5)
+(STATUS_OK, STATUS_INVALID_ARG, STATUS_NO_KERNEL, STATUS_LAUNCH_FAILED, STATUS_BAD_CONFIG,
+ STATUS_WORKSPACE_TOO_LARGE) = range(6)
+NO_ALLOC_SCRATCH_BYTES = 128 * 1024 * 1024
 
 # Every extern "C" symbol declared in include/rocm_sgemm.h.
 C_SYMBOLS = (
-    "rocm_sgemm_f32", "rocm_sgemm_f32_with_config", "rocm_sgemm_f32_strided_batched",
+    "rocm_sgemm_f32", "rocm_sgemm_f32_no_alloc", "rocm_sgemm_f32_with_config", "rocm_sgemm_f32_strided_batched",
     "rocm_sgemm_f32_strided_batched_with_config", "rocm_sgemm_nearest_config", "rocm_sgemm_find_config",
     "rocm_sgemm_find_config_batched", "rocm_sgemm_predict_us",
     "rocm_sgemm_table_size", "rocm_sgemm_table_entry", "rocm_sgemm_family_size",
@@ -105,6 +107,7 @@ def lib():
     handle.rocm_sgemm_f32.argtypes = [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_size_t,
                                       c_size_t, c_size_t, c_void_p]
     handle.rocm_sgemm_f32_with_config.argtypes = [cfg_p] + handle.rocm_sgemm_f32.argtypes
+    handle.rocm_sgemm_f32_no_alloc.argtypes = handle.rocm_sgemm_f32.argtypes
     c_float, c_ll = ctypes.c_float, ctypes.c_longlong
     handle.rocm_sgemm_f32_strided_batched.argtypes = [
         c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_ll, c_void_p, c_size_t, c_ll, c_float,
@@ -168,6 +171,16 @@ def gemm(C, A, B, M, N, K, layout_c="row_major", layout_a="row_major", layout_b=
     """C (M x N) <- A (M x K) @ B (K x N) on `stream`; buffers are dense, packed device memory."""
     _check(lib().rocm_sgemm_f32(_layout(layout_c), _layout(layout_a), _layout(layout_b),
                                 _ptr(C), _ptr(A), _ptr(B), M, N, K, _stream(stream)))
+
+
+def gemm_no_alloc(C, A, B, M, N, K, layout_c="row_major", layout_a="row_major", layout_b="row_major",
+                  stream=None):
+    """The same product as `gemm` without any device allocation: partial products of a split-K or
+    stream-K-tail config live in the library's fixed scratch array (NO_ALLOC_SCRATCH_BYTES per
+    GPU, shared by all calls on it); a problem that needs more raises SgemmError with
+    STATUS_WORKSPACE_TOO_LARGE."""
+    _check(lib().rocm_sgemm_f32_no_alloc(_layout(layout_c), _layout(layout_a), _layout(layout_b),
+                                         _ptr(C), _ptr(A), _ptr(B), M, N, K, _stream(stream)))
 
 
 def gemm_with_config(config, C, A, B, M, N, K, layout_c="row_major", layout_a="row_major",

@@ -48,6 +48,30 @@ int rocm_sgemm_f32(int          layout_c,
     return status == ROCM_SGEMM_STATUS_OK ? status : fail(status, error);
 }
 
+int rocm_sgemm_f32_no_alloc(int          layout_c,
+                            int          layout_a,
+                            int          layout_b,
+                            float*       C,
+                            const float* A,
+                            const float* B,
+                            size_t       M,
+                            size_t       N,
+                            size_t       K,
+                            void*        stream)
+{
+    using namespace rocm_sgemm::detail;
+    if(M == 0 || N == 0 || K == 0)
+    {
+        return fail(ROCM_SGEMM_STATUS_INVALID_ARG, "matrix dimensions must be positive");
+    }
+    const rocm_sgemm_config config = plan_config(M, N, K, layout_a, layout_b, layout_c);
+    gemm_problem problem{layout_c, layout_a, layout_b, C, A, B, M, N, K, 0, 0, 0, 0, 0, 0, 1, 1.0f, 0.0f};
+    problem.no_alloc = true;
+    std::string error;
+    const int   status = run_gemm(config, problem, static_cast<hipStream_t>(stream), error);
+    return status == ROCM_SGEMM_STATUS_OK ? status : fail(status, error);
+}
+
 int rocm_sgemm_f32_with_config(const rocm_sgemm_config* config,
                                int                      layout_c,
                                int                      layout_a,

@@ -4,6 +4,7 @@
 
 #include "dispatch.hpp"
 
+#include <atomic>
 #include <climits>
 #include <cmath>
 #include <cstdint>
@@ -170,6 +171,37 @@ hipError_t workspace_get(void** ptr, size_t bytes, hipStream_t stream, bool* str
     }
     buf->bytes = want;
     *ptr       = buf->ptr;
+    return hipSuccess;
+}
+
+// Scratch of the allocation-free entry point: a fixed array in device memory that exists from the
+// moment the library's code object is loaded on a GPU until the process ends (each GPU holds its
+// own copy at its own address).  On the host the array's name is only a handle for
+// hipGetSymbolAddress, not a device address; the address is looked up once per device, with that
+// device current, and only that pointer is ever handed to a kernel.
+constexpr size_t scratch_floats = ROCM_SGEMM_NO_ALLOC_SCRATCH_BYTES / sizeof(float);
+static __device__ __align__(256) float scratch[scratch_floats];
+
+constexpr int       scratch_max_devices = 64;
+std::atomic<float*> scratch_address[scratch_max_devices];
+
+hipError_t scratch_get(float** ptr)
+{
+    int        device = 0;
+    hipError_t err    = hipGetDevice(&device);
+    if(err != hipSuccess) return err;
+    if(device < 0 || device >= scratch_max_devices) return hipErrorInvalidDevice;
+    float* known = scratch_address[device].load(std::memory_order_acquire);
+    if(known == nullptr)
+    {
+        void* found = nullptr;
+        err         = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+        if(err != hipSuccess) return err;
+        if(found == nullptr) return hipErrorInvalidSymbol;
+        known = static_cast<float*>(found);
+        scratch_address[device].store(known, std::memory_order_release); // every thread finds the same value
+    }
+    *ptr = known;
     return hipSuccess;
 }
 
@@ -480,7 +512,27 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     {
         workspace_floats = static_cast<size_t>(args.tail_groups) * 2 * bm * bn;
     }
-    if(workspace_floats > 0)
+    if(workspace_floats > 0 && p.no_alloc)
+    {
+        // the fixed scratch array of this GPU: nothing is allocated, every call on the GPU shares it
+        if(workspace_floats > scratch_floats)
+        {
+            error = "this problem needs " + std::to_string(workspace_floats * sizeof(float))
+                    + " bytes of workspace for its partial products; the allocation-free entry point has "
+                    + std::to_string(scratch_floats * sizeof(float))
+                    + " (use rocm_sgemm_f32, which allocates its workspace)";
+            return ROCM_SGEMM_STATUS_WORKSPACE_TOO_LARGE;
+        }
+        float*     ws  = nullptr;
+        hipError_t err = scratch_get(&ws);
+        if(err != hipSuccess)
+        {
+            error = std::string("address of the scratch array not available: ") + hipGetErrorString(err);
+            return ROCM_SGEMM_STATUS_LAUNCH_FAILED;
+        }
+        args.partial = ws;
+    }
+    else if(workspace_floats > 0)
     {
         // the library's buffer of this stream (see workspace_get)
         void*      ws  = nullptr;

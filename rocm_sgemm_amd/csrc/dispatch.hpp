@@ -74,6 +74,9 @@ struct gemm_problem
     long long    stride_a, stride_b, stride_c;
     size_t       batch;
     float        alpha, beta;
+    /// Partial products go to the fixed scratch array of the GPU instead of an allocated workspace;
+    /// a problem that needs more than the array holds is refused.
+    bool no_alloc = false;
 };
 
 /// Validates, resolves the kernel and enqueues it.  Returns a ROCM_SGEMM_STATUS_* value and, on
