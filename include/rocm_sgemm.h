@@ -68,6 +68,12 @@ enum
  *                       (partial tiles summed by a second kernel) so that every CU has work.
  *                       0 = ask the runtime (CUs x occupancy), 1 = never, n > 1 = assume n
  *                       (tuning / testing aid)
+ *   waves_k           : replicas of the waves_m x waves_n wave grid along K (0 or 1 = none).
+ *                       Replica w multiplies the w-th part of every K-tile over the whole wave
+ *                       tile, and the partial tiles are summed through LDS before the store:
+ *                       a small macro tile (many tiles for 256 CUs) keeps a large wave tile.
+ *                       Block size = 64 * waves_m * waves_n * waves_k.  Part of the tile shape,
+ *                       like macro_m .. stages; the youngest field, hence last
  */
 typedef struct rocm_sgemm_config
 {
@@ -81,6 +87,7 @@ typedef struct rocm_sgemm_config
     int split_k;
     int group_m;
     int wave_slots;
+    int waves_k;
 } rocm_sgemm_config;
 
 /*
@@ -248,8 +255,9 @@ int rocm_sgemm_table_entry(int index, size_t* M, size_t* N, size_t* K, int* layo
                            int* layout_c, rocm_sgemm_config* out);
 
 /*
- * The precompiled tile shapes (the tuner's search space).  Only macro_m .. stages are meaningful in
- * `out`; split_k, group_m and wave_slots are launch-time parameters, returned as 1, 4 and 0.
+ * The precompiled tile shapes (the tuner's search space).  Only macro_m .. stages and waves_k are
+ * meaningful in `out`; split_k, group_m and wave_slots are launch-time parameters, returned as
+ * 1, 4 and 0.
  */
 int rocm_sgemm_family_size(void);
 int rocm_sgemm_family_entry(int index, rocm_sgemm_config* out);

@@ -31,6 +31,9 @@
 //                       `rocprofv3 --pmc <set> -- bench_float --pmc ...` (itself, one row, one
 //                       counter set at a time; this process does not touch the GPU in that phase)
 //                       and prints matrix-pipe busy %, LDS bank-conflict % and achieved HBM GB/s
+//   --host_cost         what a call costs on the host (no counterpart in the reference, whose call
+//                       is one table lookup and one launch): microseconds per
+//                       rocm_sgemm_find_config, and per enqueued call while the GPU has queue space
 //   --pmc               short run for use under rocprofv3 --pmc: 2 warm-up + 5 timed launches and
 //                       one plain 64 MiB copy kernel, whose known traffic calibrates the
 //                       FETCH_SIZE / WRITE_SIZE counters
@@ -55,6 +58,7 @@
 #include <vector>
 
 #include <hip/hip_runtime.h>
+#include <rocm_sgemm.h>
 #include <rocm_sgemm/gemm.hpp>
 
 #include "sampled_check.hpp"
@@ -100,6 +104,7 @@ struct options
     bool             vendor      = false;
     bool             pmc         = false; // child mode under rocprofv3
     bool             counters    = false; // parent mode: collect counters row by row
+    bool             host_cost   = false; // host-side cost of a call instead of the timing table
     std::vector<int> layouts; // bit 2 = A col, bit 1 = B col, bit 0 = C col; empty = all eight
 };
 
@@ -179,6 +184,8 @@ void print_usage(const char* program)
               << "  --vendor           also time rocBLAS and hipBLASLt (fp32) for context\n"
               << "  --counters         then collect rocprofv3 counters per row: MFMA busy %, LDS conflicts, HBM GB/s\n"
               << "  --pmc              short run (2 warm-up + 5 timed + a copy probe) for use under rocprofv3 --pmc\n"
+              << "  --host_cost        host microseconds per call: planning alone, and enqueueing plain / split-K /\n"
+              << "                     stream-K-tail products, one shape repeated and several shapes in turn\n"
               << "  --help             Show this help message\n"
               << "\nExamples:\n"
               << "  " << program << " --shapes 512:1024:2048\n"
@@ -811,6 +818,90 @@ int run(const options& opt)
     return failures == 0 ? 0 : 1;
 }
 
+// Host-side cost of a call.  Planning is timed on its own (host only, runs without a GPU); the
+// whole call is timed as the mean host time to enqueue a burst of calls that is short enough for
+// the GPU queue never to fill, so the host is never waiting for the device.
+int run_host_cost()
+{
+    using clock = std::chrono::steady_clock;
+    struct shape
+    {
+        size_t m, n, k;
+    };
+    const auto us_per = [](clock::time_point t0, clock::time_point t1, int n) {
+        return std::chrono::duration<double, std::micro>(t1 - t0).count() / n;
+    };
+    const auto plan_cost = [&](const char* what, const std::vector<shape>& shapes) {
+        rocm_sgemm_config cfg;
+        const int         n  = 200000;
+        const auto        t0 = clock::now();
+        for(int i = 0; i < n; ++i)
+        {
+            const shape& s = shapes[i % shapes.size()];
+            rocm_sgemm_find_config(s.m, s.n, s.k, 0, 0, 0, &cfg);
+        }
+        std::printf("host_cost plan  %-58s %8.3f us per call\n", what, us_per(t0, clock::now(), n));
+    };
+    plan_cost("table entry (4096^3)", {{4096, 4096, 4096}});
+    plan_cost("planned shape, repeated (1536 x 1200 x 900)", {{1536, 1200, 900}});
+    plan_cost("two planned shapes in turn", {{1536, 1200, 900}, {777, 2222, 1111}});
+    plan_cost("six planned shapes in turn",
+              {{1536, 1200, 900}, {777, 2222, 1111}, {640, 640, 3000}, {3000, 200, 500}, {96, 5000, 800}, {2100, 2100, 2100}});
+    std::vector<shape> many;
+    for(size_t i = 0; i < 20; ++i) many.push_back({1500 + 37 * i, 900 + 101 * i, 700 + 53 * i});
+    plan_cost("twenty planned shapes in turn (a thread remembers sixteen)", many);
+
+    int devices = 0;
+    if(hipGetDeviceCount(&devices) != hipSuccess || devices == 0)
+    {
+        (void)hipGetLastError();
+        std::printf("host_cost call  (no GPU visible: call rows skipped)\n");
+        return 0;
+    }
+    hipStream_t stream;
+    HIP_CHECK(hipStreamCreate(&stream));
+    const size_t       big = 4096 * 4096;
+    float *            dA, *dB, *dC;
+    HIP_CHECK(hipMalloc(&dA, big * sizeof(float)));
+    HIP_CHECK(hipMalloc(&dB, big * sizeof(float)));
+    HIP_CHECK(hipMalloc(&dC, big * sizeof(float)));
+    HIP_CHECK(hipMemset(dA, 0, big * sizeof(float)));
+    HIP_CHECK(hipMemset(dB, 0, big * sizeof(float)));
+    const auto call_cost = [&](const char* what, const std::vector<shape>& shapes) {
+        const int burst = 64, rounds = 20;
+        for(const shape& s : shapes) // first calls: kernels loaded, workspace of the stream in place
+            rocm_sgemm_f32(0, 0, 0, dC, dA, dB, s.m, s.n, s.k, stream);
+        HIP_CHECK(hipStreamSynchronize(stream));
+        double total = 0.0;
+        for(int r = 0; r < rounds; ++r)
+        {
+            const auto t0 = clock::now();
+            for(int i = 0; i < burst; ++i)
+            {
+                const shape& s = shapes[i % shapes.size()];
+                rocm_sgemm_f32(0, 0, 0, dC, dA, dB, s.m, s.n, s.k, stream);
+            }
+            total += us_per(t0, clock::now(), burst);
+            HIP_CHECK(hipStreamSynchronize(stream));
+        }
+        rocm_sgemm_config cfg;
+        rocm_sgemm_find_config(shapes[0].m, shapes[0].n, shapes[0].k, 0, 0, 0, &cfg);
+        std::printf("host_cost call  %-58s %8.3f us per call   (first shape: split_k %d)\n", what, total / rounds,
+                    cfg.split_k);
+    };
+    call_cost("plain product, one launch (256^3)", {{256, 256, 256}});
+    call_cost("plain product, one launch (1024^3)", {{1024, 1024, 1024}});
+    call_cost("split-K product, two launches (1024 x 1024 x 16384)", {{1024, 1024, 16384}});
+    call_cost("stream-K tail, two launches (2560^3)", {{2560, 2560, 2560}});
+    call_cost("two planned shapes in turn", {{1536, 1200, 900}, {777, 2222, 1111}});
+    call_cost("twenty planned shapes in turn", many);
+    HIP_CHECK(hipFree(dA));
+    HIP_CHECK(hipFree(dB));
+    HIP_CHECK(hipFree(dC));
+    HIP_CHECK(hipStreamDestroy(stream));
+    return 0;
+}
+
 } // namespace
 
 int main(int argc, char* argv[])
@@ -837,6 +928,8 @@ int main(int argc, char* argv[])
             opt.pmc = true, opt.warmup = 2, opt.iters = 5;
         else if(arg == "--counters")
             opt.counters = true;
+        else if(arg == "--host_cost")
+            opt.host_cost = true;
         else if(arg == "--uniform")
         {
             opt.uniform = true;
@@ -884,6 +977,10 @@ int main(int argc, char* argv[])
         return 2;
     }
 #endif
+    if(opt.host_cost)
+    {
+        return run_host_cost();
+    }
     if(opt.counters)
     {
         // Counter collection starts other processes under rocprofv3 and must not hold the GPU

@@ -29,6 +29,10 @@ BENCH_SRC = os.path.join(PKG_DIR, "benchmark", "bench_float.cpp")
 BENCH_PATH = os.path.join(PKG_DIR, "benchmark", "bench_float")
 CALLER_SRC = os.path.join(REPO_DIR, "tests", "cxx", "reference_style_caller.cpp")
 CALLER_PATH = os.path.join(REPO_DIR, "tests", "cxx", "reference_style_caller")
+# a caller that includes the reference's own host headers by path: built only where that tree is
+HEADER_CALLER_SRC = os.path.join(REPO_DIR, "tests", "cxx", "reference_header_caller.cpp")
+HEADER_CALLER_PATH = os.path.join(REPO_DIR, "tests", "cxx", "reference_header_caller")
+REFERENCE_DIR = "/root/reference"
 
 ARCH = "gfx950"
 COMMON_FLAGS = [
@@ -168,6 +172,20 @@ def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR):
                                + (proc.stdout + proc.stderr)[-4000:])
         if verbose:
             print(f"linked {CALLER_PATH}")
+        # the same with the reference's real common/matrix.hpp and common/hip_utils.hpp beside this
+        # repository's <rocm_sgemm/gemm.hpp> (nothing of the reference is copied; the binary
+        # travels with the tree to machines that do not have the reference)
+        if os.path.exists(os.path.join(REFERENCE_DIR, "common", "matrix.hpp")):
+            cmd = [hipcc(), "-std=c++17", "-O2", f"--offload-arch={ARCH}", "-Wno-unused-command-line-argument",
+                   "-I", os.path.join(REPO_DIR, "include"), "-I", REFERENCE_DIR,
+                   "-x", "hip", HEADER_CALLER_SRC, "-o", HEADER_CALLER_PATH,
+                   "-L", PKG_DIR, "-lrocm_sgemm", "-Wl,-rpath,$ORIGIN/../../rocm_sgemm_amd"]
+            proc = subprocess.run(cmd, capture_output=True, text=True)
+            if proc.returncode != 0:
+                raise RuntimeError("reference-header caller failed to build:\n"
+                                   + (proc.stdout + proc.stderr)[-4000:])
+            if verbose:
+                print(f"linked {HEADER_CALLER_PATH}")
         # the benchmark program (counterpart of the reference's bench_float), rocBLAS / hipBLASLt rows optional
         rocblas = os.path.exists("/opt/rocm/include/rocblas/rocblas.h")
         cmd = [hipcc(), "-std=c++17", "-O2", f"--offload-arch={ARCH}", "-Wno-unused-command-line-argument",

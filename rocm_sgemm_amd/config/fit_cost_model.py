@@ -22,10 +22,11 @@ import sys
 
 import numpy as np
 
-LINE = re.compile(r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) avg_ms ([\d.]+) "
+# (sweeps written before the waves_k field existed have ten integers per line)
+LINE = re.compile(r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+)(?: (\d+))? avg_ms ([\d.]+) "
                   r"min_ms ([\d.]+) tflops ([\d.]+) ok ([01])")
 KEYS = ["macro_m", "macro_n", "k_tile", "waves_m", "waves_n", "mfma", "stages", "split_k", "group_m",
-        "wave_slots"]
+        "wave_slots", "waves_k"]
 CUS = 256
 
 # name: (value compiled into csrc/planner.cpp, lower bound, upper bound)
@@ -57,7 +58,7 @@ def compiled_constants():
 
 def tail_applies(c, tiles, k_tiles, k):
     """csrc/planner.cpp tail_applies(): (applies, slots, tiles of the last wave)."""
-    waves = c["waves_m"] * c["waves_n"]
+    waves = c["waves_m"] * c["waves_n"] * max(c.get("waves_k", 1), 1)
     per_cu = 1 if waves >= 4 else 4 // max(waves, 1)
     slots = c["wave_slots"] if c["wave_slots"] > 1 else CUS * per_cu
     r = tiles % slots
@@ -70,7 +71,7 @@ def tail_applies(c, tiles, k_tiles, k):
 
 def predict(p, c, M, N, K, batch=1):
     """Restatement of csrc/planner.cpp predict_us() with the constants in `p`."""
-    waves = c["waves_m"] * c["waves_n"]
+    waves = c["waves_m"] * c["waves_n"] * max(c.get("waves_k", 1), 1)
     per_cu = 1 if waves >= 4 else 4 // max(waves, 1)
     area = (c["macro_m"] // c["waves_m"]) * (c["macro_n"] // c["waves_n"])
     eff = (p["eff_128x64"] if area >= 8192 else p["eff_64x64"] if area >= 4096
@@ -127,7 +128,8 @@ def load(patterns):
                 for line in f:
                     g = LINE.search(line)
                     if g and g.group(14) == "1":
-                        rows.append((float(g.group(11)) * 1e3, dict(zip(KEYS, map(int, g.groups()[:10])))))
+                        ints = [int(v) if v is not None else 1 for v in g.groups()[:11]]
+                        rows.append((float(g.group(12)) * 1e3, dict(zip(KEYS, ints))))
             if rows:
                 data.append((tuple(map(int, m.groups())), rows))
     return data

@@ -13,6 +13,9 @@ describe a wave32 VALU kernel (thread tiles, threads_n); an MFMA kernel is descr
                         n >= 2 -> loaded straight into a ring of n LDS stages (ragged problems
                         run the edge-masked variants of the same kernel: 16-byte loads when the
                         operand lines are 16-byte aligned, 4-byte loads otherwise)
+    waves_k             replicas of the wave grid along K: replica w multiplies the w-th part of
+                        every K-tile over the whole wave tile and the partial tiles are summed
+                        through LDS (1 = none); block size = 64 * waves_m * waves_n * waves_k
     split_k, group_m    launch-time only: K slices and tile-order band height
     wave_slots          launch-time only: 0 = deal the K range of a short last wave of tiles out
                         to all CUs (stream-K tail; slots asked from the runtime), 1 = never
@@ -38,32 +41,38 @@ PARAM_SPACE = {
     "split_k": [1, 2, 4, 8, 16],
     "group_m": [1, 2, 4, 8, 16],
     "wave_slots": [0, 1],
+    "waves_k": [1, 2, 4],
 }
 
-SHAPE_KEYS = ("macro_m", "macro_n", "k_tile", "waves_m", "waves_n", "mfma", "stages")
-CONFIG_KEYS = SHAPE_KEYS + ("split_k", "group_m", "wave_slots")
+# A tile shape (what is compiled) is the tuple of SHAPE_KEYS; a config adds the launch-time
+# parameters.  CONFIG_KEYS is the field order of struct rocm_sgemm_config, of the tuner binary's
+# command line and of its `cfg` lines: waves_k, the youngest field, sits at the end of it.
+SHAPE_KEYS = ("macro_m", "macro_n", "k_tile", "waves_m", "waves_n", "mfma", "stages", "waves_k")
+CONFIG_KEYS = SHAPE_KEYS[:7] + ("split_k", "group_m", "wave_slots", "waves_k")
 LAYOUTS = ("row_major", "col_major")
 
 
-def lds_bytes(macro_m, macro_n, k_tile, x_kc, y_kc, stages=0):
+def lds_bytes(macro_m, macro_n, k_tile, x_kc, y_kc, stages=0, waves_k=1):
     """LDS footprint; mirrors tile_config::LDS_BYTES in csrc/sgemm_mfma_kernel.hpp: padded images
-    in two stages when register-staged, unpadded images in `stages` stages when direct-to-LDS."""
+    in two stages when register-staged, unpadded images in `stages` stages when direct-to-LDS;
+    with waves along K, at least the waves_k partial-tile images (rows padded by 8 floats)."""
     if stages >= 2:
-        return stages * (macro_m + macro_n) * k_tile * 4
+        exchange = waves_k * macro_m * (macro_n + 8) * 4 if waves_k > 1 else 0
+        return max(stages * (macro_m + macro_n) * k_tile * 4, exchange)
     x = macro_m * (k_tile + 4) if x_kc else k_tile * (macro_m + 4)
     y = macro_n * (k_tile + 4) if y_kc else k_tile * (macro_n + 4)
     return 2 * (x + y) * 4
 
 
-def max_lds_bytes(macro_m, macro_n, k_tile, stages=0):
-    return max(lds_bytes(macro_m, macro_n, k_tile, a, b, stages) for a in (0, 1) for b in (0, 1))
+def max_lds_bytes(macro_m, macro_n, k_tile, stages=0, waves_k=1):
+    return max(lds_bytes(macro_m, macro_n, k_tile, a, b, stages, waves_k) for a in (0, 1) for b in (0, 1))
 
 
 def registers_per_lane(shape):
     """Estimate of registers per lane: accumulators + two fragment sets + staging + addressing.
     A pre-filter only: the build rejects any kernel the compiler has to spill."""
     macro_m, macro_n, k_tile, waves_m, waves_n, mfma = shape[:6]
-    threads = 64 * waves_m * waves_n
+    threads = 64 * waves_m * waves_n * shape[7]
     acc = (macro_m // waves_m) * (macro_n // waves_n) // 64
     tiles = (macro_m // waves_m + macro_n // waves_n) // mfma
     frags = 2 * 4 * tiles
@@ -73,14 +82,16 @@ def registers_per_lane(shape):
 
 def register_budget(shape):
     """Registers per lane available to one wave: the SIMD's 512 shared by its resident waves."""
-    waves = shape[3] * shape[4]
+    waves = shape[3] * shape[4] * shape[7]
     return REGS_PER_LANE // max(1, -(-waves // 4))
 
 
 def shape_ok(shape):
     """Constraints a tile shape must satisfy to be compiled (static_asserts of tile_config)."""
-    macro_m, macro_n, k_tile, waves_m, waves_n, mfma, stages = shape
+    macro_m, macro_n, k_tile, waves_m, waves_n, mfma, stages, waves_k = shape
     if mfma not in (32, 16):
+        return False
+    if waves_k < 1 or (waves_k > 1 and stages < 2):  # waves along K: direct-to-LDS kernels only
         return False
     if stages != 0 and not 2 <= stages <= 8:
         return False
@@ -90,16 +101,17 @@ def shape_ok(shape):
     tn = macro_n // waves_n // mfma
     if tm not in (1, 2, 4, 8) or tn not in (1, 2, 4, 8):
         return False
-    if k_tile % (8 * (64 // mfma)):  # an even number of k-blocks of 4 * (64 / mfma) depth
+    # every wave multiplies an even number of k-blocks (of 4 * (64 / mfma) depth) of a K-tile
+    if k_tile % (8 * (64 // mfma) * waves_k):
         return False
-    threads = 64 * waves_m * waves_n
+    threads = 64 * waves_m * waves_n * waves_k
     if threads > 1024:
         return False
     if (macro_m * k_tile // 4) % threads or (macro_n * k_tile // 4) % threads:
         return False
-    # the register-staged twin of a direct-to-LDS shape is compiled alongside it: both must fit
-    if max(max_lds_bytes(macro_m, macro_n, k_tile, 0),
-           max_lds_bytes(macro_m, macro_n, k_tile, stages)) > LDS_BYTES_PER_CU:
+    if waves_k > 1 and (macro_m * macro_n // 4) % threads:  # the summed tile is stored by all threads
+        return False
+    if max_lds_bytes(macro_m, macro_n, k_tile, stages, waves_k) > LDS_BYTES_PER_CU:
         return False
     if registers_per_lane(shape) > register_budget(shape):
         return False
@@ -114,56 +126,51 @@ def shape_ok(shape):
 
 def swapped(shape):
     """Shape of the kernel that serves a column-major C (operands and tile swapped)."""
-    macro_m, macro_n, k_tile, waves_m, waves_n, mfma, stages = shape
-    return (macro_n, macro_m, k_tile, waves_n, waves_m, mfma, stages)
+    macro_m, macro_n, k_tile, waves_m, waves_n, mfma, stages, waves_k = shape
+    return (macro_n, macro_m, k_tile, waves_n, waves_m, mfma, stages, waves_k)
 
 
 # Tile shapes compiled into the library (closed under `swapped`).  A deliberately small subset of
 # the valid points of PARAM_SPACE: big tiles for the compute-bound squares, small ones so that
 # skinny or small problems still produce >= 256 workgroups.
 _BASE_SHAPES = [
-    # register-staged (stages = 0)
-    (256, 256, 32, 2, 2, 32, 0),
-    (256, 256, 32, 2, 4, 32, 0),
-    (256, 128, 16, 2, 2, 32, 0),
-    (256, 128, 32, 2, 2, 32, 0),
-    (256, 128, 32, 4, 2, 32, 0),
-    (128, 128, 16, 2, 2, 32, 0),
-    (128, 128, 32, 2, 2, 32, 0),
-    (128, 64, 32, 2, 2, 32, 0),
-    (64, 64, 32, 2, 2, 32, 0),
-    (32, 32, 32, 1, 1, 32, 0),
-    # v_mfma_f32_16x16x4_f32: a 128-bit LDS read is fully used even by narrow wave tiles
-    (128, 128, 32, 2, 2, 16, 0),
-    (128, 64, 32, 2, 2, 16, 0),
-    (64, 64, 32, 2, 2, 16, 0),
-    (32, 32, 32, 1, 1, 16, 0),
     # direct-to-LDS (stages >= 2); small tiles get deeper rings, their K-tiles being short
-    (256, 256, 32, 2, 2, 32, 2),
-    (256, 256, 32, 2, 4, 32, 2),
-    (256, 128, 32, 2, 2, 32, 2),
-    (256, 128, 32, 2, 2, 32, 3),
-    (256, 128, 32, 4, 2, 32, 2),
-    (128, 128, 32, 2, 2, 32, 2),
-    (128, 128, 32, 2, 2, 32, 3),
-    (128, 128, 32, 2, 2, 32, 4),
-    (128, 64, 32, 2, 2, 32, 3),
-    (64, 64, 32, 2, 2, 32, 2),
-    (64, 64, 32, 2, 2, 32, 4),
-    (32, 32, 32, 1, 1, 32, 4),
+    (256, 256, 32, 2, 2, 32, 2, 1),
+    (256, 256, 32, 2, 4, 32, 2, 1),
+    (256, 128, 32, 2, 2, 32, 2, 1),
+    (256, 128, 32, 2, 2, 32, 3, 1),
+    (256, 128, 32, 4, 2, 32, 2, 1),
+    (128, 128, 32, 2, 2, 32, 2, 1),
+    (128, 128, 32, 2, 2, 32, 3, 1),
+    (128, 128, 32, 2, 2, 32, 4, 1),
+    (128, 64, 32, 2, 2, 32, 3, 1),
+    (64, 64, 32, 2, 2, 32, 2, 1),
+    (64, 64, 32, 2, 2, 32, 4, 1),
+    (32, 32, 32, 1, 1, 32, 4, 1),
     # K-tiles of 64: half as many pipeline steps (barriers, waits) per unit of depth, which is
     # what small tiles with few MFMAs per step are short of
-    (128, 128, 64, 2, 2, 32, 2),
-    (64, 64, 64, 2, 2, 32, 2),
-    (128, 128, 32, 2, 2, 16, 3),
-    (64, 64, 32, 2, 2, 16, 3),
-    (32, 32, 32, 1, 1, 16, 4),
+    (128, 128, 64, 2, 2, 32, 2, 1),
+    (64, 64, 64, 2, 2, 32, 2, 1),
+    # v_mfma_f32_16x16x4_f32: a 128-bit LDS read is fully used even by narrow wave tiles
+    (128, 128, 32, 2, 2, 16, 3, 1),
+    (64, 64, 32, 2, 2, 16, 3, 1),
+    (32, 32, 32, 1, 1, 16, 4, 1),
+    # waves along K: small macro tiles whose waves still own a 64 x 64 (or 64 x 32) wave tile, for
+    # problems that need many tiles to fill the GPU
+    (64, 64, 64, 1, 1, 32, 2, 4),
+    (64, 64, 64, 1, 1, 32, 3, 4),
+    (64, 32, 64, 1, 1, 32, 3, 4),
+    (128, 64, 32, 2, 1, 32, 3, 2),
+    # register-staged (stages = 0): K-tiles of 16 for very shallow problems, the one-wave tiles
+    # for one-row or one-column problems, and the classic double-buffered 128 x 128 and 64 x 64
+    # tiles as the tuner's point of comparison
+    (256, 128, 16, 2, 2, 32, 0, 1),
+    (128, 128, 16, 2, 2, 32, 0, 1),
+    (128, 128, 32, 2, 2, 32, 0, 1),
+    (64, 64, 32, 2, 2, 32, 0, 1),
+    (32, 32, 32, 1, 1, 32, 0, 1),
+    (32, 32, 32, 1, 1, 16, 0, 1),
 ]
-
-
-def base_shape(shape):
-    """The register-staged shape whose edge-masked kernel serves `shape` on ragged problems."""
-    return tuple(shape[:6]) + (0,)
 
 
 _FAMILY = None
@@ -177,9 +184,8 @@ def family():
             for t in (s, swapped(s)):
                 if not shape_ok(t):
                     raise ValueError(f"tile shape {t} violates the kernel's constraints")
-                for u in (base_shape(t), t):  # a direct-to-LDS shape needs its register-staged twin
-                    if u not in out:
-                        out.append(u)
+                if t not in out:
+                    out.append(t)
         _FAMILY = out
     return list(_FAMILY)
 
@@ -220,4 +226,5 @@ DEFAULT_CONFIG = {
     "split_k": 1,
     "group_m": 4,
     "wave_slots": 0,
+    "waves_k": 1,
 }

@@ -36,7 +36,7 @@ import space  # noqa: E402
 
 LAYOUT_ALIASES = {"r": 0, "row_major": 0, "c": 1, "col_major": 1}
 SWEEP_LINE = re.compile(
-    r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) avg_ms ([\d.]+) min_ms ([\d.]+) "
+    r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) avg_ms ([\d.]+) min_ms ([\d.]+) "
     r"tflops ([\d.]+) ok ([01])")
 
 
@@ -187,7 +187,7 @@ class Tuner:
                  f"({2.0 * M * N * K / best['avg_ms'] * 1e-9:.1f} TFLOP/s, {len(trials)} trials)")
         return {"M": M, "N": N, "K": K, "layout": layout, "config": best["config"],
                 "avg_time_ms": best["avg_ms"], "evaluations": len(trials),
-                "memory_used_bytes": space.max_lds_bytes(*shape[:3], shape[6]),
+                "memory_used_bytes": space.max_lds_bytes(*shape[:3], shape[6], shape[7]),
                 "space_coverage_percent": round(100.0 * len({tuple(t['config'][k] for k in space.SHAPE_KEYS) for t in trials}) / max(1, len(self.shapes)), 1)}
 
     def tune_all(self, sizes, layouts, baselines_for=None):

@@ -4,10 +4,10 @@
 // a trial is a plain library call - rocm_sgemm_f32_with_config - because every tile shape of the
 // search space is compiled into librocm_sgemm; nothing is compiled at run time.
 //
-//   tuner M N K macro_m macro_n k_tile waves_m waves_n mfma stages split_k group_m wave_slots A B C [iters] [warmup]
+//   tuner M N K macro_m macro_n k_tile waves_m waves_n mfma stages split_k group_m wave_slots waves_k A B C [iters] [warmup]
 //       layouts: 0 = row_major, 1 = col_major.  Prints "time: <avg> ms  min: <min> ms ...".
 //   tuner --sweep M N K A B C [--iters n] [--warmup n] [--splits a,b,..] [--groups a,b,..] [--slots a,b,..]
-//       one line per (tile shape, split_k, group_m):  "cfg <10 ints> avg_ms <..> min_ms <..> tflops <..> ok <0|1>"
+//       one line per (tile shape, split_k, group_m):  "cfg <11 ints> avg_ms <..> min_ms <..> tflops <..> ok <0|1>"
 //
 // Inputs are uniform[-1, 1) from a fixed xorshift stream; every trial is checked on 256 sampled
 // entries against an fp64 dot product so that a mis-tuned config can never enter the table.
@@ -186,7 +186,7 @@ int usage()
 {
     std::fprintf(stderr,
                  "usage: tuner M N K macro_m macro_n k_tile waves_m waves_n mfma stages split_k group_m "
-                 "wave_slots A B C [iters] [warmup]\n"
+                 "wave_slots waves_k A B C [iters] [warmup]\n"
                  "       tuner --sweep M N K A B C [--iters n] [--warmup n] [--splits a,b] "
                  "[--groups a,b]\n");
     return 2;
@@ -236,9 +236,9 @@ int main(int argc, char** argv)
                     if(!rocm_sgemm_config_supported(&cfg, p.lc, p.la, p.lb)) continue;
                     const timing t = run_trial(p, cfg, iters, warmup);
                     if(!t.launched) continue;
-                    std::printf("cfg %d %d %d %d %d %d %d %d %d %d avg_ms %.4f min_ms %.4f tflops %.2f ok %d\n",
+                    std::printf("cfg %d %d %d %d %d %d %d %d %d %d %d avg_ms %.4f min_ms %.4f tflops %.2f ok %d\n",
                                 cfg.macro_m, cfg.macro_n, cfg.k_tile, cfg.waves_m, cfg.waves_n,
-                                cfg.mfma, cfg.stages, cfg.split_k, cfg.group_m, cfg.wave_slots, t.avg_ms,
+                                cfg.mfma, cfg.stages, cfg.split_k, cfg.group_m, cfg.wave_slots, cfg.waves_k, t.avg_ms,
                                 t.min_ms,
                                 flops / (t.avg_ms * 1e-3) * 1e-12, t.correct ? 1 : 0);
                     std::fflush(stdout);
@@ -249,7 +249,7 @@ int main(int argc, char** argv)
         return 0;
     }
 
-    if(argc < 17)
+    if(argc < 18)
     {
         return usage();
     }
@@ -260,10 +260,10 @@ int main(int argc, char** argv)
     rocm_sgemm_config cfg{std::atoi(argv[4]), std::atoi(argv[5]), std::atoi(argv[6]),
                           std::atoi(argv[7]), std::atoi(argv[8]), std::atoi(argv[9]),
                           std::atoi(argv[10]), std::atoi(argv[11]), std::atoi(argv[12]),
-                          std::atoi(argv[13])};
-    p.la = std::atoi(argv[14]), p.lb = std::atoi(argv[15]), p.lc = std::atoi(argv[16]);
-    const int iters  = argc > 17 ? std::atoi(argv[17]) : 20;
-    const int warmup = argc > 18 ? std::atoi(argv[18]) : 3;
+                          std::atoi(argv[13]), std::atoi(argv[14])};
+    p.la = std::atoi(argv[15]), p.lb = std::atoi(argv[16]), p.lc = std::atoi(argv[17]);
+    const int iters  = argc > 18 ? std::atoi(argv[18]) : 20;
+    const int warmup = argc > 19 ? std::atoi(argv[19]) : 3;
     if(!rocm_sgemm_config_supported(&cfg, p.lc, p.la, p.lb))
     {
         std::fprintf(stderr, "unsupported config: %s\n", rocm_sgemm_last_error());

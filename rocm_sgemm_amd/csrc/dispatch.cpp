@@ -24,7 +24,7 @@ namespace detail
 
 struct tile_shape
 {
-    int macro_m, macro_n, k_tile, waves_m, waves_n, mfma, stages;
+    int macro_m, macro_n, k_tile, waves_m, waves_n, mfma, stages, waves_k;
 };
 
 struct kernel_family_row
@@ -32,7 +32,7 @@ struct kernel_family_row
     tile_shape shape;
     // [X depth-contiguous][Y depth-contiguous][variant]
     //   0: full tiles (direct-to-LDS when stages >= 2)
-    //   1: edge-masked, register-staged (for a direct-to-LDS shape: its stages = 0 twin's, unused)
+    //   1: edge-masked, register-staged (stages = 0 shapes; null otherwise)
     //   2: edge-masked direct-to-LDS, 16-byte loads (null for stages = 0 shapes)
     //   3: edge-masked direct-to-LDS, 4-byte loads (null for stages = 0 shapes)
     launch_fn launch[2][2][4];
@@ -43,13 +43,14 @@ struct kernel_family_row
 namespace
 {
 
-const kernel_family_row* find_shape(int bm, int bn, int bk, int wm, int wn, int mfma, int stages)
+const kernel_family_row* find_shape(int bm, int bn, int bk, int wm, int wn, int mfma, int stages, int waves_k)
 {
+    const int wk = waves_k < 1 ? 1 : waves_k; // 0 (a config written before the field existed) = none
     for(int i = 0; i < kernel_family_size; ++i)
     {
         const tile_shape& s = kernel_family[i].shape;
         if(s.macro_m == bm && s.macro_n == bn && s.k_tile == bk && s.waves_m == wm
-           && s.waves_n == wn && s.mfma == mfma && s.stages == stages)
+           && s.waves_n == wn && s.mfma == mfma && s.stages == stages && s.waves_k == wk)
         {
             return &kernel_family[i];
         }
@@ -61,8 +62,8 @@ std::string describe(const rocm_sgemm_config& c)
 {
     return "macro " + std::to_string(c.macro_m) + "x" + std::to_string(c.macro_n) + ", k_tile "
            + std::to_string(c.k_tile) + ", waves " + std::to_string(c.waves_m) + "x"
-           + std::to_string(c.waves_n) + ", mfma " + std::to_string(c.mfma) + ", stages "
-           + std::to_string(c.stages);
+           + std::to_string(c.waves_n) + (c.waves_k > 1 ? "x" + std::to_string(c.waves_k) : std::string())
+           + ", mfma " + std::to_string(c.mfma) + ", stages " + std::to_string(c.stages);
 }
 
 bool is_layout(int v)
@@ -255,7 +256,7 @@ void family_entry(int index, rocm_sgemm_config* out)
 {
     const tile_shape& s = kernel_family[index].shape;
     *out                = rocm_sgemm_config{s.macro_m, s.macro_n, s.k_tile, s.waves_m, s.waves_n,
-                                            s.mfma, s.stages, 1, 4, 0};
+                                            s.mfma, s.stages, 1, 4, 0, s.waves_k};
 }
 
 bool config_supported(const rocm_sgemm_config& c, int layout_c, int layout_a, int layout_b,
@@ -273,8 +274,8 @@ bool config_supported(const rocm_sgemm_config& c, int layout_c, int layout_a, in
     }
     const bool swap = layout_c == ROCM_SGEMM_COL_MAJOR;
     const kernel_family_row* row
-        = swap ? find_shape(c.macro_n, c.macro_m, c.k_tile, c.waves_n, c.waves_m, c.mfma, c.stages)
-               : find_shape(c.macro_m, c.macro_n, c.k_tile, c.waves_m, c.waves_n, c.mfma, c.stages);
+        = swap ? find_shape(c.macro_n, c.macro_m, c.k_tile, c.waves_n, c.waves_m, c.mfma, c.stages, c.waves_k)
+               : find_shape(c.macro_m, c.macro_n, c.k_tile, c.waves_m, c.waves_n, c.mfma, c.stages, c.waves_k);
     if(row == nullptr)
     {
         error = "No kernel available for the requested configuration and layout (" + describe(c)
@@ -401,7 +402,7 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     // accumulation registers and cost the 256-accumulator shapes their register budget.
     const bool scaled = !(p.alpha == 1.0f && p.beta == 0.0f);
 
-    const kernel_family_row* row = find_shape(bm, bn, c.k_tile, wm, wn, c.mfma, c.stages);
+    const kernel_family_row* row = find_shape(bm, bn, c.k_tile, wm, wn, c.mfma, c.stages, c.waves_k);
     if(row == nullptr)
     {
         error = "No kernel available for the requested configuration and layout (" + describe(c)

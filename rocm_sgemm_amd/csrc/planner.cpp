@@ -7,6 +7,7 @@
 #include <climits>
 #include <cmath>
 #include <limits>
+#include <vector>
 
 namespace rocm_sgemm
 {
@@ -28,12 +29,36 @@ bool key_less(const tuned_entry& e, size_t m, size_t n, size_t k, int la, int lb
     return e.layout_c < lc;
 }
 
-double log2_distance(size_t m1, size_t n1, size_t k1, size_t m2, size_t n2, size_t k2)
+// Distance between two problem sizes: sum of squared log2 ratios (the reference's measure).  The
+// logarithms of the built-in table's sizes are computed once per process, those of a problem once
+// per lookup: a lookup scans the table up to three times.
+struct log_size
 {
-    const double dm = std::log2(static_cast<double>(m1)) - std::log2(static_cast<double>(m2));
-    const double dn = std::log2(static_cast<double>(n1)) - std::log2(static_cast<double>(n2));
-    const double dk = std::log2(static_cast<double>(k1)) - std::log2(static_cast<double>(k2));
+    double m, n, k;
+};
+
+log_size logs_of(size_t m, size_t n, size_t k)
+{
+    return log_size{std::log2(static_cast<double>(m)), std::log2(static_cast<double>(n)),
+                    std::log2(static_cast<double>(k))};
+}
+
+double log2_distance(const log_size& a, const log_size& b)
+{
+    const double dm = a.m - b.m, dn = a.n - b.n, dk = a.k - b.k;
     return dm * dm + dn * dn + dk * dk;
+}
+
+const log_size* builtin_logs()
+{
+    static const std::vector<log_size> logs = [] {
+        std::vector<log_size> v;
+        v.reserve(tuned_table_size > 0 ? tuned_table_size : 1);
+        for(int i = 0; i < tuned_table_size; ++i)
+            v.push_back(logs_of(tuned_table[i].m, tuned_table[i].n, tuned_table[i].k));
+        return v;
+    }();
+    return logs.data();
 }
 
 } // namespace
@@ -77,8 +102,11 @@ const rocm_sgemm_config& select_config(const tuned_entry*       table,
     // others run the masked kernels with 4-byte loads, and the best tile shapes of the two kinds
     // differ.  So entries of the problem's own kind are searched first (the
     // reference's table holds powers of two only and never meets the distinction).
-    double best      = std::numeric_limits<double>::max();
-    int    best_idx  = -1;
+    double          best     = std::numeric_limits<double>::max();
+    int             best_idx = -1;
+    const log_size  here     = logs_of(m, n, k);
+    const log_size* known    = table == tuned_table ? builtin_logs() : nullptr; // else a caller's own table
+    const auto      entry_logs = [&](int i) { return known ? known[i] : logs_of(table[i].m, table[i].n, table[i].k); };
     const auto whole = [](size_t a, size_t b, size_t c) { return a % 4 == 0 && b % 4 == 0 && c % 4 == 0; };
     for(int same_kind = 1; same_kind >= 0 && best_idx < 0; --same_kind)
     {
@@ -88,7 +116,7 @@ const rocm_sgemm_config& select_config(const tuned_entry*       table,
             if(e.layout_a == la && e.layout_b == lb && e.layout_c == lc
                && (!same_kind || whole(e.m, e.n, e.k) == whole(m, n, k)))
             {
-                const double d = log2_distance(m, n, k, e.m, e.n, e.k);
+                const double d = log2_distance(here, entry_logs(i));
                 if(d < best)
                 {
                     best     = d;
@@ -104,8 +132,7 @@ const rocm_sgemm_config& select_config(const tuned_entry*       table,
     // Nearest size of any layout.
     for(int i = 0; i < table_size; ++i)
     {
-        const tuned_entry& e = table[i];
-        const double       d = log2_distance(m, n, k, e.m, e.n, e.k);
+        const double d = log2_distance(here, entry_logs(i));
         if(d < best)
         {
             best     = d;
@@ -149,7 +176,7 @@ void fit_split(rocm_sgemm_config& c, size_t m, size_t n, size_t k, size_t batch)
 bool tail_applies(const rocm_sgemm_config& c, long long tiles, long long k_tiles, size_t k, long long cus,
                   long long* slots_out, long long* r_out)
 {
-    const int       waves  = c.waves_m * c.waves_n;
+    const int       waves  = c.waves_m * c.waves_n * (c.waves_k > 1 ? c.waves_k : 1);
     const int       per_cu = waves >= 4 ? 1 : 4 / (waves < 1 ? 1 : waves); // workgroups that fill a CU's four SIMDs
     const long long slots  = c.wave_slots > 1 ? c.wave_slots : cus * per_cu;
     const long long r      = tiles % slots;
@@ -174,7 +201,7 @@ bool tail_applies(const rocm_sgemm_config& c, long long tiles, long long k_tiles
 // mainly the ordering matters.
 double predict_us(const rocm_sgemm_config& c, size_t m, size_t n, size_t k, size_t batch)
 {
-    const int    waves     = c.waves_m * c.waves_n;
+    const int    waves     = c.waves_m * c.waves_n * (c.waves_k > 1 ? c.waves_k : 1);
     const int    per_cu    = waves >= 4 ? 1 : 4 / (waves < 1 ? 1 : waves);
     const double wave_area = static_cast<double>(c.macro_m / c.waves_m) * (c.macro_n / c.waves_n);
     double       eff = wave_area >= 8192 ? 0.996 : wave_area >= 4096 ? 0.970 : wave_area >= 2048 ? 0.954 : 0.926;
@@ -237,7 +264,9 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
 }
 
 // Planning costs a few microseconds for a problem that is not a table entry; callers usually
-// repeat a shape, so every thread remembers its last answer (the tables never change).
+// work through a handful of shapes again and again (the layers of a model, the steps of a
+// factorisation), so every thread remembers its last sixteen answers (the tables never change).
+// Sixteen slots, replaced in turn: a lookup is a scan of at most sixteen keys.
 rocm_sgemm_config plan_config(size_t m, size_t n, size_t k, int la, int lb, int lc, size_t batch)
 {
     struct memo
@@ -246,14 +275,23 @@ rocm_sgemm_config plan_config(size_t m, size_t n, size_t k, int la, int lb, int 
         int               la = -1, lb = -1, lc = -1;
         rocm_sgemm_config config{};
     };
-    thread_local memo last;
-    if(last.m != m || last.n != n || last.k != k || last.batch != batch || last.la != la || last.lb != lb
-       || last.lc != lc)
+    constexpr int          slots = 16;
+    thread_local memo      remembered[slots];
+    thread_local int       used = 0, next = 0;
+    for(int i = 0; i < used; ++i)
     {
-        last.config = plan_uncached(m, n, k, la, lb, lc, batch < 1 ? 1 : batch);
-        last.m = m, last.n = n, last.k = k, last.batch = batch, last.la = la, last.lb = lb, last.lc = lc;
+        const memo& e = remembered[i];
+        if(e.m == m && e.n == n && e.k == k && e.batch == batch && e.la == la && e.lb == lb && e.lc == lc)
+        {
+            return e.config;
+        }
     }
-    return last.config;
+    memo& e  = remembered[next];
+    e.config = plan_uncached(m, n, k, la, lb, lc, batch < 1 ? 1 : batch);
+    e.m = m, e.n = n, e.k = k, e.batch = batch, e.la = la, e.lb = lb, e.lc = lc;
+    next = next + 1 == slots ? 0 : next + 1;
+    used = used < slots ? used + 1 : slots;
+    return e.config;
 }
 
 namespace
@@ -280,7 +318,9 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     // split_k 1, 2, 4 and 8; the cheapest of them replaces the nearest entry's config only if
     // the model expects it to be at least 4 % faster (about the model's own error).
     const auto aligned_kind = [](size_t a, size_t b, size_t c) { return a % 4 == 0 && b % 4 == 0 && c % 4 == 0; };
-    constexpr int max_candidates = 4;
+    constexpr int   max_candidates = 4;
+    const log_size  here  = logs_of(m, n, k);
+    const log_size* known = builtin_logs();
     int           idx[max_candidates];
     double        dist[max_candidates];
     int           count = 0;
@@ -292,7 +332,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
         {
             continue;
         }
-        const double d = log2_distance(m, n, k, e.m, e.n, e.k);
+        const double d = log2_distance(here, known[i]);
         int          pos = count < max_candidates ? count : max_candidates;
         while(pos > 0 && d < dist[pos - 1]) --pos; // strict: the first of equals stays first
         if(pos >= max_candidates) continue;
@@ -334,7 +374,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
         {
             if(split > 1 && k_tiles < 2LL * split) break; // at least two K-tiles per slice
             consider(rocm_sgemm_config{s.macro_m, s.macro_n, s.k_tile, s.waves_m, s.waves_n, s.mfma, s.stages,
-                                       split, 4, 0});
+                                       split, 4, 0, s.waves_k});
         }
     }
     return best;

@@ -36,6 +36,13 @@
 // layout needs is done by choosing which four values one 128-bit LDS read delivers:
 //   depth-contiguous image [row][k] : one read = 4 consecutive k of ONE row  -> feeds 4 MFMA k-steps
 //   row-contiguous image   [k][row] : one read = 4 consecutive rows of ONE k -> feeds 4 MFMA tiles
+// Waves along K (WK > 1): the WM x WN wave grid is replicated WK times and replica w multiplies
+// only the k-blocks [w * NKB / WK, (w + 1) * NKB / WK) of every K-tile, over the whole wave tile;
+// the WK partial tiles are summed through LDS before the store.  A 64 x 64 macro tile with WK = 4
+// gives every wave a 64 x 64 wave tile (four independent accumulator tiles, one LDS read per four
+// MFMAs) where the plain 2 x 2 wave grid gives it one 32 x 32 tile (a chain of dependent MFMAs and
+// one read per two): small macro tiles, which small and skinny problems need to fill 256 CUs,
+// then run the inner loop of a large one.
 // An MI x MI MFMA (MI = 32: 32x32x2, MI = 16: 16x16x4) takes its row/column from lane % MI and its
 // k from the lane group h = lane / MI (2 or 4 groups).  Inside every "k-block" of 4 * (64 / MI)
 // k values (8 or 16), MFMA step r (0..3) multiplies k = 4*h + r; X and Y use the same assignment,
@@ -99,7 +106,7 @@ struct gemm_args
 };
 
 template<int BM_, int BN_, int BK_, int WM_, int WN_, int MI_, bool X_KC_, bool Y_KC_, bool EDGE_, int NS_ = 0,
-         int DG_ = 4>
+         int DG_ = 4, int WK_ = 1>
 struct tile_config
 {
     static constexpr int  BM   = BM_;
@@ -118,8 +125,11 @@ struct tile_config
     // element's own and serves operands whose lines start anywhere (odd leading dimensions,
     // unaligned pointers, any K), at four times the number of load instructions.
     static constexpr int DG = DG_;
+    // Waves along K: the wave grid is replicated WK times, replica w works on the w-th part of the
+    // k-blocks of every K-tile, and the partial tiles are summed through LDS at the end.
+    static constexpr int WK = WK_;
 
-    static constexpr int NT  = 64 * WM * WN; // threads per workgroup
+    static constexpr int NT  = 64 * WM * WN * WK; // threads per workgroup
     static constexpr int WTM = BM / WM; // wave tile
     static constexpr int WTN = BN / WN;
     static constexpr int TM  = WTM / MI; // MFMA tiles per wave
@@ -127,6 +137,7 @@ struct tile_config
     static constexpr int ACC = MI * MI / 64; // accumulator registers per MFMA tile
     static constexpr int KB  = 4 * (64 / MI); // depth of a k-block: 4 MFMA steps
     static constexpr int NKB = BK / KB; // k-blocks per K-tile
+    static constexpr int NKBW = NKB / WK; // k-blocks of a K-tile one wave multiplies
 
     // Interleave width of a row-contiguous operand (tiles fed by one LDS read).
     static constexpr int VM = TM >= 4 ? 4 : TM;
@@ -146,7 +157,13 @@ struct tile_config
     static constexpr int Y_SIZE = Y_KC ? BN * LDY : BK * LDY;
     static constexpr int STAGE  = X_SIZE + Y_SIZE;
     static constexpr int STAGES = DTL ? NS : 2;
-    static constexpr int LDS_BYTES = STAGES * STAGE * 4;
+    // WK > 1: after the main loop every wave-grid replica leaves its partial tile in LDS as a
+    // BM x BN row-major image with rows EX_LD floats apart (the 8 floats of padding put the two
+    // rows a 32 x 32 MFMA tile's lane groups write at once 32 banks apart).
+    static constexpr int EX_LD     = BN + 8;
+    static constexpr int EX_FLOATS = WK > 1 ? WK * BM * EX_LD : 0;
+    static constexpr int LDS_FLOATS = STAGES * STAGE > EX_FLOATS ? STAGES * STAGE : EX_FLOATS;
+    static constexpr int LDS_BYTES = LDS_FLOATS * 4;
 
     // Swizzle of a depth-contiguous direct-to-LDS image: rows of BK floats, CPR 16-byte chunks
     // each, RPL rows per 64-bank line.
@@ -160,7 +177,10 @@ struct tile_config
 
     static_assert(MI == 32 || MI == 16, "MFMA tile is 32x32x2 or 16x16x4");
     static_assert(BM % (MI * WM) == 0 && BN % (MI * WN) == 0, "wave tile must be a multiple of the MFMA tile");
-    static_assert(BK % (2 * KB) == 0, "K-tile holds an even number of k-blocks");
+    static_assert(WK >= 1 && NKB % WK == 0 && (NKB / WK) % 2 == 0,
+                  "every wave multiplies an even number of k-blocks of a K-tile");
+    static_assert(WK == 1 || DTL, "waves along K exist for the direct-to-LDS kernels only");
+    static_assert((BM * BN / 4) % NT == 0, "the summed tile must divide evenly among the threads");
     static_assert(DG == 4 || (DG == 1 && DTL && EDGE), "single-float loads exist for the masked direct-to-LDS kernel only");
     static_assert((BM * BK / 4) % NT == 0 && (BN * BK / 4) % NT == 0, "chunks must divide evenly");
     static_assert(TM == 1 || TM == 2 || TM % 4 == 0, "TM in {1,2,4,8,...}");
@@ -520,26 +540,29 @@ template<class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args args)
 {
     constexpr int  BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
-    constexpr int  TM = Cfg::TM, TN = Cfg::TN, NT = Cfg::NT, NKB = Cfg::NKB;
+    constexpr int  TM = Cfg::TM, TN = Cfg::TN, NT = Cfg::NT, NKB = Cfg::NKBW, WK = Cfg::WK;
     constexpr bool X_KC = Cfg::X_KC, Y_KC = Cfg::Y_KC, EDGE = Cfg::EDGE, DTL = Cfg::DTL;
     constexpr int  VM = Cfg::VM, VN = Cfg::VN, MI = Cfg::MI, ACC = Cfg::ACC;
     constexpr int  NS = Cfg::STAGES;
     typedef float acc_t __attribute__((ext_vector_type(ACC)));
 
-    __shared__ __attribute__((aligned(16))) float lds[NS * Cfg::STAGE];
+    __shared__ __attribute__((aligned(16))) float lds[Cfg::LDS_FLOATS];
 
     const int tid  = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int lane = tid % 64;
     const int h    = lane / MI; // lane group: selects k inside an MFMA
     const int c    = lane % MI; // row (X operand) / column (Y operand) inside an MFMA tile
-    const int wm0  = (wave / Cfg::WN) * Cfg::WTM;
-    const int wn0  = (wave % Cfg::WN) * Cfg::WTN;
+    const int wk   = wave / (Cfg::WM * Cfg::WN); // replica of the wave grid = part of every K-tile
+    const int wmn  = wave % (Cfg::WM * Cfg::WN);
+    const int wm0  = (wmn / Cfg::WN) * Cfg::WTM;
+    const int wn0  = (wmn % Cfg::WN) * Cfg::WTN;
+    const int kb0  = wk * NKB; // first k-block of a K-tile this wave multiplies
 
     // Workgroup -> one or two segments (tile, K range).
     //   ids below tail_begin (all ids when there is no tail): one segment.  With split_k > 1 every
-    //                    tile has split_k slices; the slice is the slow index, so the tile order
-    //                    (and its L2 locality) is the same inside every slice.
+    //                    tile has split_k slices; the slice is the slow index of the sequence that
+    //                    is dealt out to the XCDs in contiguous chunks.
     //   ids from tail_begin on: workgroup g of the stream-K tail owns K-tiles [g * tail_per,
     //                    (g + 1) * tail_per) of the tail tiles laid end to end, i.e. a piece of one
     //                    tile and possibly the beginning of the next.
@@ -695,25 +718,29 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
     {
         const int u = h ^ dma_x::swz(c);
         impl::static_for<0, NKB>([&](auto kb) {
-            xs_base[decltype(kb)::value] = (wm0 + c) * BK + (((decltype(kb)::value * KBC) ^ u) * 4);
+            xs_base[decltype(kb)::value] = (wm0 + c) * BK + ((((kb0 + decltype(kb)::value) * KBC) ^ u) * 4);
         });
     }
     if constexpr(DTL && Y_KC)
     {
         const int u = h ^ dma_y::swz(c);
         impl::static_for<0, NKB>([&](auto kb) {
-            ys_base[decltype(kb)::value] = (wn0 + c) * BK + (((decltype(kb)::value * KBC) ^ u) * 4);
+            ys_base[decltype(kb)::value] = (wn0 + c) * BK + ((((kb0 + decltype(kb)::value) * KBC) ^ u) * 4);
         });
     }
     float fx[2][TM][4];
     float fy[2][TN][4];
+    // depth offset of this wave's k-blocks inside an image that is not addressed through the
+    // swizzle table above: depth lines of a row-contiguous image, floats of an unswizzled row
+    const int x_koff = (X_KC ? (DTL ? 0 : 1) : Cfg::LDX) * (kb0 * Cfg::KB);
+    const int y_koff = (Y_KC ? (DTL ? 0 : 1) : Cfg::LDY) * (kb0 * Cfg::KB);
     auto  read_item = [&](int q, int slot, int buf, int kb) { // LDS stage buf -> fragment set slot
         const float* sx = lds + buf * Cfg::STAGE;
         if(q < NRX)
-            impl::read_one<X_KC, DTL, TM, VM, Cfg::LDX, MI>(q, fx[slot], sx, xs_base, wm0, kb, h, c);
+            impl::read_one<X_KC, DTL, TM, VM, Cfg::LDX, MI>(q, fx[slot], sx + x_koff, xs_base, wm0, kb, h, c);
         else
-            impl::read_one<Y_KC, DTL, TN, VN, Cfg::LDY, MI>(q - NRX, fy[slot], sx + Cfg::X_SIZE, ys_base,
-                                                            wn0, kb, h, c);
+            impl::read_one<Y_KC, DTL, TN, VN, Cfg::LDY, MI>(q - NRX, fy[slot], sx + Cfg::X_SIZE + y_koff,
+                                                            ys_base, wn0, kb, h, c);
     };
 
     for(int seg = 0; seg < nseg; ++seg)
@@ -725,15 +752,28 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
         k_begin     = (max(run0, u * k_tiles) - u * k_tiles) * BK;
         k_end       = min(args.depth, (min(run1, (u + 1) * k_tiles) - u * k_tiles) * BK);
     }
+    else if(args.split_k > 1)
+    {
+        // K slices: the whole (slice, tile) sequence, slice-major, is cut into one contiguous chunk
+        // per XCD, so an XCD works on the tiles of one slice (or of a few): its workgroups share
+        // one K range of both operands in its L2 instead of the whole depth of a few panels
+        const int seq = detail::xcd_chunked_index(blockIdx.x, tiles * args.split_k);
+        slice         = seq / tiles;
+        wg            = seq - slice * tiles;
+        k_begin       = slice * args.k_slice;
+        k_end         = min(args.depth, k_begin + args.k_slice);
+    }
     else
     {
-        slice   = blockIdx.x / tiles;
-        wg      = blockIdx.x - slice * tiles;
-        k_begin = slice * args.k_slice;
-        k_end   = min(args.depth, k_begin + args.k_slice);
+        wg      = blockIdx.x;
+        k_begin = 0;
+        k_end   = args.depth;
     }
     {
-        const detail::tile_coord tc = detail::map_workgroup(wg, args.grid_m, args.grid_n, args.group_m);
+        const detail::tile_coord tc
+            = !tail && args.split_k > 1
+                  ? detail::banded_tile(wg, args.grid_m, args.grid_n, args.group_m < 1 ? 1 : args.group_m)
+                  : detail::map_workgroup(wg, args.grid_m, args.grid_n, args.group_m);
         m0 = tc.tile_m * BM;
         n0 = tc.tile_n * BN;
     }
@@ -898,6 +938,60 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
         P   = args.P + batch * args.stride_p;
         ldp = args.ldp, row_base = m0, col_base = n0, row_end = args.rows, col_end = args.cols;
     }
+    if constexpr(WK > 1)
+    {
+        // Waves along K: every replica of the wave grid holds a partial of the whole macro tile.
+        // Each leaves it in LDS as a row-major BM x BN image; then the workgroup sums the images in
+        // replica order (fixed, so the result does not depend on timing) and stores whole rows,
+        // four adjacent columns per thread.
+        constexpr int EX_LD = Cfg::EX_LD;
+        __syncthreads(); // every wave is done with the stages: the images reuse their memory
+        float* image = lds + wk * (BM * EX_LD);
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+#pragma unroll
+            for(int v = 0; v < ACC; ++v)
+            {
+                const int r = wm0 + impl::tile_index<X_KC, VM, MI>(i, impl::acc_row<MI>(v, h_e));
+#pragma unroll
+                for(int j = 0; j < TN; ++j)
+                    image[r * EX_LD + wn0 + impl::tile_index<Y_KC, VN, MI>(j, c_e)] = acc[i][j][v];
+            }
+        __syncthreads();
+#pragma unroll
+        for(int g = 0; g < BM * BN / 4 / NT; ++g)
+        {
+            const int q = g * NT + tid;
+            const int r = q / (BN / 4);
+            const int n = (q % (BN / 4)) * 4;
+            f32x4     o = *reinterpret_cast<const f32x4*>(lds + r * EX_LD + n);
+#pragma unroll
+            for(int w = 1; w < WK; ++w)
+                o += *reinterpret_cast<const f32x4*>(lds + w * (BM * EX_LD) + r * EX_LD + n);
+            const int row = row_base + r;
+            const int col = col_base + n;
+            float*    dst = P + static_cast<size_t>(row) * ldp + col;
+            if constexpr(!EDGE)
+            {
+                *reinterpret_cast<f32x4*>(dst) = o;
+            }
+            else if(row < row_end)
+            {
+                if(col + 3 < col_end)
+                {
+                    *reinterpret_cast<f32x4_e*>(dst) = o;
+                }
+                else
+                {
+                    if(col < col_end) dst[0] = o.x;
+                    if(col + 1 < col_end) dst[1] = o.y;
+                    if(col + 2 < col_end) dst[2] = o.z;
+                }
+            }
+        }
+    }
+    else
+    {
 #pragma unroll
     for(int i = 0; i < TM; ++i)
     {
@@ -970,6 +1064,7 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
             }
         }
     }
+    } // WK == 1
     if(seg + 1 < nseg)
     {
         // the next segment refills the LDS stages: every wave must be done reading them

@@ -321,21 +321,26 @@ def test_tile_order_rejects_out_of_range():
 # ---- search space model and generator ----------------------------------------------------------
 
 def test_space_constraints():
-    assert space.shape_ok((256, 256, 16, 2, 2, 32, 0))
-    assert not space.shape_ok((256, 256, 64, 2, 2, 32, 0))  # 2 stages of 256x(64+4)x2 floats > 160 KB
-    assert not space.shape_ok((96, 128, 16, 2, 2, 32, 0))  # wave tile not a multiple of 32
-    assert not space.shape_ok((128, 128, 24, 2, 2, 32, 0))  # odd number of k-blocks
-    assert not space.shape_ok((128, 128, 32, 1, 1, 32, 0))  # register budget
+    assert space.shape_ok((256, 256, 16, 2, 2, 32, 0, 1))
+    assert not space.shape_ok((256, 256, 64, 2, 2, 32, 0, 1))  # 2 stages of 256x(64+4)x2 floats > 160 KB
+    assert not space.shape_ok((96, 128, 16, 2, 2, 32, 0, 1))  # wave tile not a multiple of 32
+    assert not space.shape_ok((128, 128, 24, 2, 2, 32, 0, 1))  # odd number of k-blocks
+    assert not space.shape_ok((128, 128, 32, 1, 1, 32, 0, 1))  # register budget
     assert space.lds_bytes(256, 256, 16, 1, 0) == 2 * (256 * 20 + 16 * 260) * 4
     # direct-to-LDS: unpadded images, `stages` of them
     assert space.lds_bytes(256, 256, 32, 1, 0, 2) == 2 * 512 * 32 * 4
-    assert space.shape_ok((256, 256, 32, 2, 4, 32, 2))
-    assert not space.shape_ok((256, 256, 32, 2, 4, 32, 3))  # 3 x 64 KB > 160 KB
-    assert not space.shape_ok((128, 128, 32, 2, 2, 32, 1))  # a ring has at least two stages
-    assert all(space.max_lds_bytes(*s[:3], s[6]) <= space.LDS_BYTES_PER_CU for s in space.family())
+    assert space.shape_ok((256, 256, 32, 2, 4, 32, 2, 1))
+    assert not space.shape_ok((256, 256, 32, 2, 4, 32, 3, 1))  # 3 x 64 KB > 160 KB
+    assert not space.shape_ok((128, 128, 32, 2, 2, 32, 1, 1))  # a ring has at least two stages
+    assert all(space.max_lds_bytes(*s[:3], s[6], s[7]) <= space.LDS_BYTES_PER_CU for s in space.family())
     assert set(space.family()) <= set(space.all_valid_shapes())
-    # ragged problems run the register-staged twin of a direct-to-LDS shape: it must be compiled
-    assert all(space.base_shape(s) in space.family() for s in space.family())
+    # waves along K: direct-to-LDS only, an even number of k-blocks per wave, <= 1024 threads,
+    # and LDS for the partial-tile images
+    assert space.shape_ok((64, 64, 64, 1, 1, 32, 2, 4))
+    assert not space.shape_ok((64, 64, 64, 1, 1, 32, 0, 4))
+    assert not space.shape_ok((64, 64, 32, 1, 1, 32, 2, 4))  # one k-block per wave
+    assert not space.shape_ok((256, 256, 32, 2, 4, 32, 2, 2))  # 2 x 256 x 264 floats > 160 KB
+    assert space.lds_bytes(64, 64, 64, 1, 0, 2, 4) == 4 * 64 * 72 * 4
 
 
 def test_generator_outputs(tmp_path):
@@ -350,9 +355,8 @@ def test_generator_outputs(tmp_path):
     j.write_text(json.dumps(doc))
     srcs = generate_config.generate(str(j), str(tmp_path / "gen"))
     assert len(srcs) == 4 * len(space.family())
-    # a direct-to-LDS shape compiles a full-tile kernel and two masked direct-to-LDS kernels of its
-    # own (16-byte and 4-byte loads) and borrows the register-staged edge kernel of its
-    # stages = 0 twin
+    # a direct-to-LDS shape compiles a full-tile kernel and two masked kernels (16-byte and 4-byte
+    # loads), a register-staged shape a full-tile and one masked kernel
     dtl = [p for p in srcs if "_s2_" in os.path.basename(p)]
     assert dtl and all(open(p).read().count("launch_kernel<") == 3 for p in dtl)
     staged = [p for p in srcs if "_s" not in os.path.basename(p).split("_m")[1]]
@@ -362,7 +366,9 @@ def test_generator_outputs(tmp_path):
     assert table.index("{64u, 256u, 128u, 0, 0, 0") < table.index("{512u, 256u, 128u, 1, 0, 1")
     ktab = (tmp_path / "gen" / "kernel_table.inc").read_text()
     assert f"kernel_family_size = {len(space.family())}" in ktab
-    assert ktab.count("nullptr") == 8 * sum(1 for f in space.family() if f[6] == 0)
+    # null slots: the two masked direct-to-LDS variants of a register-staged shape, the
+    # register-staged variant of a direct-to-LDS shape; four orientations each
+    assert ktab.count("nullptr") == 4 * sum(2 if f[6] == 0 else 1 for f in space.family())
     bad = dict(cfg, macro_m=96)
     doc["configurations"][0]["config"] = bad
     j.write_text(json.dumps(doc))
@@ -403,9 +409,9 @@ def _fake_runner(best_shape, best_group):
                 for sp in splits:
                     for g in groups:
                         ms = 1.0 if (s == best_shape and sp == 1) else 2.0
-                        lines.append("cfg " + " ".join(map(str, s + (sp, g, 0)))
+                        lines.append("cfg " + " ".join(map(str, s[:7] + (sp, g, 0, s[7])))
                                      + f" avg_ms {ms:.4f} min_ms {ms:.4f} tflops 1.00 ok 1")
-            lines.append("cfg 32 32 32 1 1 32 0 1 4 0 avg_ms 0.0100 min_ms 0.0100 tflops 9.00 ok 0")
+            lines.append("cfg 32 32 32 1 1 32 0 1 4 0 1 avg_ms 0.0100 min_ms 0.0100 tflops 9.00 ok 0")
             return _FakeProc("\n".join(lines))
         cfg = dict(zip(space.CONFIG_KEYS, map(int, cmd[4:4 + len(space.CONFIG_KEYS)])))
         shape = tuple(cfg[k] for k in space.SHAPE_KEYS)
@@ -415,7 +421,7 @@ def _fake_runner(best_shape, best_group):
 
 
 def test_tuner_driver_finds_planted_optimum_and_merges(tmp_path):
-    best_shape = (256, 128, 32, 4, 2, 32, 2)
+    best_shape = (256, 128, 32, 4, 2, 32, 2, 1)
     run, calls = _fake_runner(best_shape, 8)
     t = tune.Tuner("tuner", budget=400, runner=run, verbose=False)
     rec = t.tune_problem(4096, 4096, 4096, (0, 1, 0))
@@ -434,14 +440,14 @@ def test_tuner_driver_finds_planted_optimum_and_merges(tmp_path):
 
 
 def test_tuner_budget_and_split_candidates():
-    run, calls = _fake_runner((128, 128, 32, 2, 2, 32, 0), 4)
+    run, calls = _fake_runner((128, 128, 32, 2, 2, 32, 0, 1), 4)
     t = tune.Tuner("tuner", budget=5, runner=run, verbose=False)
     rec = t.tune_problem(1024, 1024, 16384, (0, 0, 0))
     # the family sweep is one process and always complete; the budget only stops phase 2
     assert not any(c[1] != "--sweep" for c in calls)
-    assert tuple(rec["config"][k] for k in space.SHAPE_KEYS) == (128, 128, 32, 2, 2, 32, 0)
-    assert tune.split_candidates((256, 256, 16, 2, 2, 32, 0), 8192, 8192, 8192) == [1]
-    assert 4 in tune.split_candidates((256, 256, 16, 2, 2, 32, 0), 1024, 1024, 16384)
+    assert tuple(rec["config"][k] for k in space.SHAPE_KEYS) == (128, 128, 32, 2, 2, 32, 0, 1)
+    assert tune.split_candidates((256, 256, 16, 2, 2, 32, 0, 1), 8192, 8192, 8192) == [1]
+    assert 4 in tune.split_candidates((256, 256, 16, 2, 2, 32, 0, 1), 1024, 1024, 16384)
     assert tune.parse_layouts(["r,c,r", "col_major,row_major,col_major"]) == [(0, 1, 0), (1, 0, 1)]
     assert tune.parse_sizes(["128,4096,4096"]) == [(128, 4096, 4096)]
 
