@@ -221,6 +221,11 @@ struct timing
     int    iters = 0;
 };
 
+// Warm-up is by count AND by time: after an idle gap the GPU takes tens of milliseconds of
+// sustained work to reach its full clock, so at least `warm_ms` of back-to-back launches precede
+// the timed ones whatever `warmup` says (0 under rocprofv3 --pmc, where every launch is costly).
+double min_warm_ms = 40.0;
+
 template<class Launch>
 timing time_launches(Launch&& launch, hipStream_t stream, int warmup, int iters, double flops)
 {
@@ -230,6 +235,20 @@ timing time_launches(Launch&& launch, hipStream_t stream, int warmup, int iters,
     for(int i = 0; i < warmup; ++i)
         launch();
     HIP_CHECK(hipStreamSynchronize(stream));
+    double warmed_ms = 0.0;
+    for(int batch = 4; warmed_ms < min_warm_ms;)
+    {
+        HIP_CHECK(hipEventRecord(e0, stream));
+        for(int i = 0; i < batch; ++i)
+            launch();
+        HIP_CHECK(hipEventRecord(e1, stream));
+        HIP_CHECK(hipEventSynchronize(e1));
+        float ms = 0;
+        HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+        warmed_ms += ms;
+        const double left = (min_warm_ms - warmed_ms) * batch / (ms > 1e-3f ? ms : 1e-3f);
+        batch             = left < 1.0 ? 1 : (left > 4096.0 ? 4096 : static_cast<int>(left));
+    }
     timing t;
     t.min_ms            = std::numeric_limits<double>::max();
     double sum_ms       = 0, sum_tf = 0;
@@ -633,8 +652,9 @@ int run(const options& opt)
     HIP_CHECK(hipGetDeviceProperties(&prop, 0));
     std::printf("device: %s %s, %d CUs, %d MHz; peak used for pct_peak: %.1f TFLOP/s (dense FP32 matrix)\n",
                 prop.name, prop.gcnArchName, prop.multiProcessorCount, prop.clockRate / 1000, peak_tflops);
-    std::printf("protocol: %d warm-up + %d timed launches per row, one event pair per launch; inputs: %s\n",
-                opt.warmup, opt.iters,
+    std::printf("protocol: %d warm-up launches (and at least %.0f ms of them) + %d timed launches per row, one event "
+                "pair per launch, each waited for; inputs: %s\n",
+                opt.warmup, min_warm_ms, opt.iters,
                 opt.identity_b ? "A uniform[-1,1), B = identity"
                                : (opt.uniform ? "uniform[-1,1)" : "cyclic {1.025,1.05,1.075,1.1,1.0}"));
     print_header();
@@ -925,7 +945,7 @@ int main(int argc, char* argv[])
         else if(arg == "--vendor")
             opt.vendor = true;
         else if(arg == "--pmc")
-            opt.pmc = true, opt.warmup = 2, opt.iters = 5;
+            opt.pmc = true, opt.warmup = 2, opt.iters = 5, min_warm_ms = 0.0;
         else if(arg == "--counters")
             opt.counters = true;
         else if(arg == "--host_cost")

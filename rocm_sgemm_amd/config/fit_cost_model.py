@@ -6,11 +6,13 @@ by a small analytic model of a launch's duration.  Its structure is fixed (see `
 restates the C++ `predict_us` of csrc/planner.cpp term by term); its constants are fitted here.
 
 Input: logs of `tuner --sweep M N K a b c --splits 1,2,4,8 --groups 4` (one line per timed config:
-`cfg <10 ints> avg_ms .. min_ms .. tflops .. ok 1`), one file per problem, named
-`sweep_<M>_<N>_<K>*.log`.  The fit minimises the squared error of log(time), weighting each config
+`cfg <11 ints> avg_ms .. min_ms .. tflops .. ok 1`), one file per problem, named
+`sweep_<M>_<N>_<K>*.log`.  `--collect DIR` writes them: it runs the tuner binary (on a GPU) on
+every problem of fit_problems.txt, the list the compiled constants were fitted on.  The fit minimises the squared error of log(time), weighting each config
 by exp(-(t / t_best - 1) / 0.25) so that the ordering among a problem's fast configs matters most.
 
-usage: fit_cost_model.py 'logs/sweep_*.log' [...]      prints the fitted constants, the quality of
+usage: fit_cost_model.py --collect DIR [--iters n]     sweeps the problems of fit_problems.txt into DIR
+       fit_cost_model.py 'DIR/sweep_*.log' [...]       prints the fitted constants, the quality of
                                                         picking configs by the model (chosen / best
                                                         time per problem) and a 3-fold check
 """
@@ -117,6 +119,10 @@ def predict(p, c, M, N, K, batch=1):
 
 def load(patterns):
     """[((M, N, K), [(microseconds, config dict), ...]), ...] from sweep logs."""
+    import os
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import space
+    family = set(space.family())
     data = []
     for pattern in patterns:
         for path in sorted(glob.glob(pattern)):
@@ -127,9 +133,11 @@ def load(patterns):
             with open(path) as f:
                 for line in f:
                     g = LINE.search(line)
-                    if g and g.group(14) == "1":
+                    if g and g.group(15) == "1":
                         ints = [int(v) if v is not None else 1 for v in g.groups()[:11]]
-                        rows.append((float(g.group(12)) * 1e3, dict(zip(KEYS, ints))))
+                        cfg = dict(zip(KEYS, ints))
+                        if tuple(cfg[k] for k in space.SHAPE_KEYS) in family:  # shapes since dropped
+                            rows.append((float(g.group(12)) * 1e3, cfg))
             if rows:
                 data.append((tuple(map(int, m.groups())), rows))
     return data
@@ -137,7 +145,8 @@ def load(patterns):
 
 def planner_candidate(c):
     """The shapes the planner lets the model choose from (csrc/planner.cpp plan_config)."""
-    return c["stages"] >= 2 and c["mfma"] == 32 and c["macro_m"] >= 64 and c["macro_n"] >= 64
+    return (c["stages"] >= 2 and c["mfma"] == 32
+            and ((c["macro_m"] >= 64 and c["macro_n"] >= 64) or c.get("waves_k", 1) > 1))
 
 
 def pick_quality(p, data):
@@ -168,10 +177,33 @@ def fit(data):
     return dict(zip(NAMES, least_squares(residuals, x0, bounds=(lo, hi)).x))
 
 
+def collect(out_dir, iters=20):
+    """Sweeps every problem of fit_problems.txt with the tuner binary (needs a GPU)."""
+    import os
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(here, "fit_problems.txt")) as f:
+        problems = [tuple(map(int, line.split())) for line in f if line.strip() and not line.startswith("#")]
+    for i, (M, N, K) in enumerate(problems):
+        log = os.path.join(out_dir, f"sweep_{M}_{N}_{K}.log")
+        cmd = [os.path.join(here, "tuner"), "--sweep", str(M), str(N), str(K), "0", "0", "0", "--iters",
+               str(iters), "--splits", "1,2,4,8", "--groups", "4"]
+        with open(log, "w") as out:
+            rc = subprocess.run(cmd, stdout=out, stderr=subprocess.STDOUT, timeout=600).returncode
+        print(f"[{i + 1}/{len(problems)}] {M} x {N} x {K}: rc {rc}", flush=True)
+        if rc != 0:
+            return rc
+    return 0
+
+
 def main(argv):
     if len(argv) < 2:
         print(__doc__)
         return 2
+    if argv[1] == "--collect":
+        iters = int(argv[argv.index("--iters") + 1]) if "--iters" in argv else 20
+        return collect(argv[2], iters)
     data = load(argv[1:])
     if not data:
         print("no sweep logs matched", file=sys.stderr)

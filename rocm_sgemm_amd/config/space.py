@@ -33,7 +33,7 @@ NUM_XCD = 8
 PARAM_SPACE = {
     "macro_m": [32, 64, 128, 256],
     "macro_n": [32, 64, 128, 256],
-    "k_tile": [16, 32, 64],
+    "k_tile": [16, 32, 64, 128],
     "waves_m": [1, 2, 4],
     "waves_n": [1, 2, 4],
     "mfma": [32, 16],
@@ -157,10 +157,10 @@ _BASE_SHAPES = [
     (32, 32, 32, 1, 1, 16, 4, 1),
     # waves along K: small macro tiles whose waves still own a 64 x 64 (or 64 x 32) wave tile, for
     # problems that need many tiles to fill the GPU
-    (64, 64, 64, 1, 1, 32, 2, 4),
     (64, 64, 64, 1, 1, 32, 3, 4),
     (64, 32, 64, 1, 1, 32, 3, 4),
     (128, 64, 32, 2, 1, 32, 3, 2),
+    (64, 64, 128, 1, 1, 32, 2, 4),
     # register-staged (stages = 0): K-tiles of 16 for very shallow problems, the one-wave tiles
     # for one-row or one-column problems, and the classic double-buffered 128 x 128 and 64 x 64
     # tiles as the tuner's point of comparison

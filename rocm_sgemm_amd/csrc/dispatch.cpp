@@ -443,21 +443,24 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     // Full tiles of 16-byte aligned lines: the kernel without masks (direct-to-LDS if the shape
     // has one, whose loads fault on a misaligned address).  Anything else: the edge-masked kernel.
     const bool to_workspace  = split > 1 || scaled; // the kernel then writes packed partials only
-    const bool in_aligned    = aligned16(p.A) && aligned16(p.B) && args.ldx % 4 == 0 && args.ldy % 4 == 0
-                               && (p.batch == 1 || (args.stride_x % 4 == 0 && args.stride_y % 4 == 0));
+    // An operand can travel 16 bytes per lane when every line of it starts on a 16-byte boundary
+    // (a misaligned load of that size faults) and, if it is stored depth-contiguous, its rows end
+    // on one (whole 16-byte pieces beyond K are dropped; one straddling the end of a row could
+    // not be).  Otherwise it travels 4 bytes per lane, which needs no alignment.
+    const bool x_aligned = aligned16(args.X) && args.ldx % 4 == 0 && (p.batch == 1 || args.stride_x % 4 == 0);
+    const bool y_aligned = aligned16(args.Y) && args.ldy % 4 == 0 && (p.batch == 1 || args.stride_y % 4 == 0);
     const bool out_aligned   = to_workspace
                                || (aligned16(p.C) && args.ldp % 4 == 0
                                    && (p.batch == 1 || args.stride_p % 4 == 0));
-    const bool full = args.rows % bm == 0 && args.cols % bn == 0 && args.depth % bk == 0 && in_aligned
-                      && out_aligned;
-    // Everything else runs an edge-masked kernel.  A direct-to-LDS shape: with 16-byte loads when
-    // the operand lines are 16-byte aligned (a misaligned load of that size faults) and the rows
-    // of a depth-contiguous operand end on a 16-byte boundary (whole 16-byte pieces beyond K are
-    // dropped; one straddling the end could not be), otherwise with 4-byte loads, which need no
-    // alignment.  A register-staged shape: its own edge-masked kernel.
-    const bool      k_whole  = args.depth % 4 == 0 || (!x_kc && !y_kc);
+    const bool full = args.rows % bm == 0 && args.cols % bn == 0 && args.depth % bk == 0 && x_aligned
+                      && y_aligned && out_aligned;
+    // Full tiles of 16-byte aligned lines: the kernel without masks.  Anything else runs an
+    // edge-masked kernel: a direct-to-LDS shape the one with 16-byte loads if both operands allow
+    // them, else the one with 4-byte loads; a register-staged shape its own.
+    const bool      x_wide   = x_aligned && (!x_kc || args.depth % 4 == 0);
+    const bool      y_wide   = y_aligned && (!y_kc || args.depth % 4 == 0);
     const launch_fn masked   = row->launch[x_kc ? 1 : 0][y_kc ? 1 : 0][2];
-    const int       variant  = full ? 0 : (masked == nullptr ? 1 : (in_aligned && k_whole ? 2 : 3));
+    const int       variant  = full ? 0 : (masked == nullptr ? 1 : (x_wide && y_wide ? 2 : 3));
     launch_fn       fn       = row->launch[x_kc ? 1 : 0][y_kc ? 1 : 0][variant];
 
     // Stream-K tail.  The matrix pipes of the GPU are saturated by W workgroups (one per CU for

@@ -314,7 +314,8 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     // reference's answer, but the log-distance rule is blind to how a tile shape divides this
     // problem's M and N and to how many tiles that leaves for 256 CUs.  So the cost model also
     // prices the configs of the four nearest entries of the same layouts and kind, and every
-    // direct-to-LDS tile shape of the family with 32 x 32 MFMAs and tiles of at least 64 x 64 at
+    // direct-to-LDS tile shape of the family with 32 x 32 MFMAs and tiles of at least 64 x 64 (or
+    // smaller ones with waves along K, which keep a large wave tile) at
     // split_k 1, 2, 4 and 8; the cheapest of them replaces the nearest entry's config only if
     // the model expects it to be at least 4 % faster (about the model's own error).
     const auto aligned_kind = [](size_t a, size_t b, size_t c) { return a % 4 == 0 && b % 4 == 0 && c % 4 == 0; };
@@ -368,7 +369,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     {
         rocm_sgemm_config s{};
         family_entry(i, &s);
-        if(s.stages < 2 || s.mfma != 32 || s.macro_m < 64 || s.macro_n < 64) continue;
+        if(s.stages < 2 || s.mfma != 32 || ((s.macro_m < 64 || s.macro_n < 64) && s.waves_k <= 1)) continue;
         const long long k_tiles = static_cast<long long>((k + s.k_tile - 1) / s.k_tile);
         for(int split = 1; split <= 8; split *= 2)
         {

@@ -25,9 +25,11 @@
 //     16-byte pieces of a depth-contiguous row at or beyond K are rejected lane by lane (they
 //     arrive as zeros too) and the stores are predicated, which covers ragged M, N and K as long
 //     as the rows of a depth-contiguous operand end on a 16-byte boundary (K a multiple of 4).
-//     With DG == 1 the same kernel moves 4 bytes per lane (buffer_load_dword ... lds) into the
-//     same LDS images, which lifts every alignment requirement: odd leading dimensions, unaligned
-//     pointers, any K.
+//     With DGX == 1 (DGY == 1) the same kernel moves X (Y) 4 bytes per lane (buffer_load_dword
+//     ... lds) into the same LDS image, which lifts every alignment requirement on that operand:
+//     odd leading dimension, unaligned pointer, any K.  The granularity is chosen per operand: in
+//     a row-major 1000 x 3000 x 777 product only A's lines (777 floats) are misaligned, B's (3000
+//     floats) still travel 16 bytes per lane.
 //   register-staged (NS == 0; the alternative for shapes without an LDS ring):
 //     HBM --128-bit buffer loads--> registers (one K-tile ahead)
 //         --128-bit ds_write, same orientation as in memory--> LDS (two stages)
@@ -106,7 +108,7 @@ struct gemm_args
 };
 
 template<int BM_, int BN_, int BK_, int WM_, int WN_, int MI_, bool X_KC_, bool Y_KC_, bool EDGE_, int NS_ = 0,
-         int DG_ = 4, int WK_ = 1>
+         int DGX_ = 4, int DGY_ = 4, int WK_ = 1>
 struct tile_config
 {
     static constexpr int  BM   = BM_;
@@ -124,7 +126,8 @@ struct tile_config
     // needs 16-byte aligned global addresses; 1 (buffer_load_dword ... lds) needs none beyond the
     // element's own and serves operands whose lines start anywhere (odd leading dimensions,
     // unaligned pointers, any K), at four times the number of load instructions.
-    static constexpr int DG = DG_;
+    static constexpr int DGX = DGX_; // X operand
+    static constexpr int DGY = DGY_; // Y operand
     // Waves along K: the wave grid is replicated WK times, replica w works on the w-th part of the
     // k-blocks of every K-tile, and the partial tiles are summed through LDS at the end.
     static constexpr int WK = WK_;
@@ -170,10 +173,9 @@ struct tile_config
     static constexpr int CPR = BK / 4;
     static constexpr int RPL = 64 / BK > 0 ? 64 / BK : 1;
 
-    // Pieces each thread moves per K-tile: 128-bit chunks, or DG floats on the direct-to-LDS path.
-    static constexpr int PIECE = DTL ? DG : 4;
-    static constexpr int CX    = BM * BK / PIECE / NT;
-    static constexpr int CY    = BN * BK / PIECE / NT;
+    // Pieces each thread moves per K-tile: 128-bit chunks, or DGX / DGY floats on the direct-to-LDS path.
+    static constexpr int CX = BM * BK / (DTL ? DGX : 4) / NT;
+    static constexpr int CY = BN * BK / (DTL ? DGY : 4) / NT;
 
     static_assert(MI == 32 || MI == 16, "MFMA tile is 32x32x2 or 16x16x4");
     static_assert(BM % (MI * WM) == 0 && BN % (MI * WN) == 0, "wave tile must be a multiple of the MFMA tile");
@@ -181,7 +183,8 @@ struct tile_config
                   "every wave multiplies an even number of k-blocks of a K-tile");
     static_assert(WK == 1 || DTL, "waves along K exist for the direct-to-LDS kernels only");
     static_assert((BM * BN / 4) % NT == 0, "the summed tile must divide evenly among the threads");
-    static_assert(DG == 4 || (DG == 1 && DTL && EDGE), "single-float loads exist for the masked direct-to-LDS kernel only");
+    static_assert((DGX == 4 || DGX == 1) && (DGY == 4 || DGY == 1), "16-byte or 4-byte pieces");
+    static_assert((DGX == 4 && DGY == 4) || (DTL && EDGE), "single-float loads exist for the masked direct-to-LDS kernel only");
     static_assert((BM * BK / 4) % NT == 0 && (BN * BK / 4) % NT == 0, "chunks must divide evenly");
     static_assert(TM == 1 || TM == 2 || TM % 4 == 0, "TM in {1,2,4,8,...}");
     static_assert(TN == 1 || TN == 2 || TN % 4 == 0, "TN in {1,2,4,8,...}");
@@ -655,9 +658,9 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
     // direct-to-LDS path: every access of a full tile is inside the operand, so there the buffer
     // range is left wide open and costs no per-tile arithmetic; the edge-masked variant passes the
     // distance to the operand's end, beyond which the hardware delivers zeros
-    constexpr int DG = Cfg::DG;
-    using dma_x = impl::dma_map<X_KC, BM, BK, NT, DG>;
-    using dma_y = impl::dma_map<Y_KC, BN, BK, NT, DG>;
+    constexpr int DGX = Cfg::DGX, DGY = Cfg::DGY;
+    using dma_x = impl::dma_map<X_KC, BM, BK, NT, DGX>;
+    using dma_y = impl::dma_map<Y_KC, BN, BK, NT, DGY>;
     // per-lane offsets: piece i uses entry i % PERIOD (plus the uniform i * STEP * ld)
     constexpr int NVX = !DTL ? 1 : (dma_x::PERIOD < CX ? dma_x::PERIOD : CX);
     constexpr int NVY = !DTL ? 1 : (dma_y::PERIOD < CY ? dma_y::PERIOD : CY);
@@ -692,8 +695,8 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
                 if constexpr(EDGE && X_KC)
                     voff = x_dpos[i % NVX] < k_rem ? voff : impl::dma_reject;
                 const float* tile = x_tile(t);
-                impl::dma_load<DG>(tile, EDGE ? min(bytes_to(tile, x_end), impl::dma_max_bytes) : 0x7FFFFFFFu,
-                                   voff, soff, st + (i * NT + wave * 64) * DG);
+                impl::dma_load<DGX>(tile, EDGE ? min(bytes_to(tile, x_end), impl::dma_max_bytes) : 0x7FFFFFFFu,
+                                    voff, soff, st + (i * NT + wave * 64) * DGX);
             }
             else
             {
@@ -703,8 +706,8 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
                 if constexpr(EDGE && Y_KC)
                     voff = y_dpos[j % NVY] < k_rem ? voff : impl::dma_reject;
                 const float* tile = y_tile(t);
-                impl::dma_load<DG>(tile, EDGE ? min(bytes_to(tile, y_end), impl::dma_max_bytes) : 0x7FFFFFFFu,
-                                   voff, soff, st + Cfg::X_SIZE + (j * NT + wave * 64) * DG);
+                impl::dma_load<DGY>(tile, EDGE ? min(bytes_to(tile, y_end), impl::dma_max_bytes) : 0x7FFFFFFFu,
+                                    voff, soff, st + Cfg::X_SIZE + (j * NT + wave * 64) * DGY);
             }
         }
     };
@@ -842,7 +845,7 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
     // must land before this iteration's barrier, so they are issued as early as two per slot allow.
     constexpr int DENSE_KBS    = impl::max_int(1, (NMOVE + 2 * SLOTS - 1) / (2 * SLOTS));
     constexpr int MOVE_KBS     = RSG_MOVE_SPREAD ? NKB - 1
-                                 : (DTL && DG == 1) ? (NS >= 3 || DENSE_KBS > NKB - 1 ? NKB - 1 : DENSE_KBS)
+                                 : (DTL && (DGX == 1 || DGY == 1)) ? (NS >= 3 || DENSE_KBS > NKB - 1 ? NKB - 1 : DENSE_KBS)
                                                     : 1;
     constexpr int MOVE_SLOTS   = MOVE_KBS * SLOTS;
     int           cur          = 0; // stage of K-tile t

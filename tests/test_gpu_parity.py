@@ -87,8 +87,11 @@ def test_all_ones_gives_k():
 # (direct-to-LDS where the shape has one) kernels; 352 = 11 K-tiles of 32 wraps every LDS ring.
 # (300, 260, 128), (36, 68, 192) and (300, 260, 100) have leading dimensions that are multiples of
 # 4 in every layout: they run the masked direct-to-LDS kernels, the last with a ragged last K-tile.
+# (300, 257, 100) and (257, 300, 100) have one odd dimension: depending on the layout one operand's
+# lines are 16-byte aligned and the other's are not (16-byte loads for one, 4-byte for the other).
 EDGE_SHAPES = [(1, 1, 1), (33, 65, 17), (255, 257, 129), (300, 260, 100), (64, 64, 64),
-               (512, 256, 96), (256, 512, 352), (257, 511, 263), (300, 260, 128), (36, 68, 192)]
+               (512, 256, 96), (256, 512, 352), (257, 511, 263), (300, 260, 128), (36, 68, 192),
+               (300, 257, 100), (257, 300, 100)]
 
 
 @pytest.mark.parametrize("la,lb,lc", ALL_LAYOUTS, ids=LAYOUT_IDS)
@@ -450,7 +453,8 @@ def test_nothing_outside_an_operand_reaches_the_result(la, lb, lc):
     picks = family
     for fam in picks:
         cfg = dict(fam.as_dict(), split_k=1, group_m=2, wave_slots=1)
-        for (M, N, K, off) in [(132, 68, 100, 1024), (260, 264, 36, 512), (131, 67, 70, 1021)]:
+        for (M, N, K, off) in [(132, 68, 100, 1024), (260, 264, 36, 512), (131, 67, 70, 1021),
+                               (132, 67, 100, 1024), (131, 68, 36, 512)]:
             _announce("inf_arena", cfg, M, N, K, off, la, lb, lc)
             A, B, C = int_matrices(rng, M, N, K)
             a, b = oracle.to_storage(A, la), oracle.to_storage(B, lb)

@@ -87,7 +87,8 @@ def _py_plan(table, M, N, K, a, b, c):
     """Restatement of the planning rule around the library's own cost model: table entries are
     returned as they are; otherwise the nearest entry's config, unless one of the four nearest
     entries of the same layouts and kind (split_k fitted first) or one of the larger direct-to-LDS
-    tile shapes at split_k 1, 2, 4 or 8 is predicted at least 4 % faster."""
+    tile shapes (or smaller ones with waves along K) at split_k 1, 2, 4 or 8 is predicted at least
+    4 % faster."""
     nearest = _py_select(table, M, N, K, a, b, c).as_dict()
     if any(key == (M, N, K, a, b, c) for key, _ in table):
         return nearest
@@ -104,7 +105,7 @@ def _py_plan(table, M, N, K, a, b, c):
     nearest_us = best_us = rs.predict_us(best, M, N, K)
     candidates = [_fit_split(table[i][1].as_dict(), M, N, K) for _, i in pool[:4]]
     for fam in rs.family():
-        if fam.stages < 2 or fam.mfma != 32 or fam.macro_m < 64 or fam.macro_n < 64:
+        if fam.stages < 2 or fam.mfma != 32 or ((fam.macro_m < 64 or fam.macro_n < 64) and fam.waves_k <= 1):
             continue
         k_tiles = -(-K // fam.k_tile)
         for split in (1, 2, 4, 8):
@@ -210,16 +211,20 @@ def test_whole_tile_and_ragged_problems_look_up_entries_of_their_own_kind():
 
 
 def test_inherited_split_k_is_fitted_to_the_problem():
-    """256 x 256 x 16384 inherits split_k = 8 from the 1024 x 1024 x 16384 entry, which would make
-    32 workgroups of 128 x 128 tiles on 256 CUs; it must run unsplit instead (the stream-K tail
-    then deals the K range out to every CU).  A table entry itself is never altered."""
+    """256 x 256 x 16384 inherits 128 x 128 tiles with split_k = 8 from the 1024 x 1024 x 16384
+    entry, which would put 32 workgroups on 256 CUs.  The plan must fill the GPU instead: either
+    unsplit with the stream-K tail dealing the K range out to every CU, or with tiles small enough
+    that tiles x split_k covers at least half the CUs.  A table entry itself is never altered."""
     table = {k: c.as_dict() for k, c in rs.table()}
     entry = table.get((1024, 1024, 16384, 0, 0, 0))
     if entry is None or entry["split_k"] <= 1:
         pytest.skip("the shipped table has no split-K entry at 1024 x 1024 x 16384")
     assert rs.find_config(1024, 1024, 16384).as_dict() == entry
     small = rs.find_config(256, 256, 16384).as_dict()
-    assert small["split_k"] == 1 and small["wave_slots"] == 0
+    groups = -(-256 // small["macro_m"]) * -(-256 // small["macro_n"]) * small["split_k"]
+    assert (small["split_k"] == 1 and small["wave_slots"] == 0) or groups >= 128, small
+    nearest = rs.nearest_config(256, 256, 16384).as_dict()
+    assert rs.predict_us(small, 256, 256, 16384) < rs.predict_us(nearest, 256, 256, 16384)
 
 
 def test_every_table_config_has_a_kernel_for_its_layout():
