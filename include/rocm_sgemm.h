@@ -73,7 +73,14 @@ enum
  *                       tile, and the partial tiles are summed through LDS before the store:
  *                       a small macro tile (many tiles for 256 CUs) keeps a large wave tile.
  *                       Block size = 64 * waves_m * waves_n * waves_k.  Part of the tile shape,
- *                       like macro_m .. stages; the youngest field, hence last
+ *                       like macro_m .. stages
+ *   partial_sums      : who adds up the partial tiles of a K split or a stream-K tail.
+ *                       1 = a second kernel; 2 = the GEMM launch itself, whenever it can (the wave
+ *                       that completes a tile's counter adds the tile's parts up: no second
+ *                       launch, but one wave reads all parts of its share of the tile);
+ *                       0 = the library decides (in the launch for products of at least 8 GFLOP
+ *                       whose waves have at most 48 KB to add up, else a second kernel).
+ *                       The result is the same bit for bit either way (same order of addition)
  */
 typedef struct rocm_sgemm_config
 {
@@ -88,6 +95,7 @@ typedef struct rocm_sgemm_config
     int group_m;
     int wave_slots;
     int waves_k;
+    int partial_sums;
 } rocm_sgemm_config;
 
 /*
@@ -223,7 +231,7 @@ int rocm_sgemm_nearest_config(size_t M, size_t N, size_t K, int layout_a, int la
  * (dropped in favour of the stream-K tail when the grid would stay well under one workgroup per
  * CU, reduced when it would exceed four per CU); the cost model below then prices that config,
  * those of the next three nearest entries and the larger direct-to-LDS tile shapes of the family
- * at split_k 1, 2, 4 and 8, and the cheapest replaces the nearest entry's config if it is
+ * at split_k 1, 2, 3, 4, 6 and 8, and the cheapest replaces the nearest entry's config if it is
  * expected to be at least 4 % faster (distance in log size says nothing about how a tile shape
  * divides M and N or how many tiles are left for 256 CUs).  Host-only, needs no GPU.
  */
@@ -256,8 +264,8 @@ int rocm_sgemm_table_entry(int index, size_t* M, size_t* N, size_t* K, int* layo
 
 /*
  * The precompiled tile shapes (the tuner's search space).  Only macro_m .. stages and waves_k are
- * meaningful in `out`; split_k, group_m and wave_slots are launch-time parameters, returned as
- * 1, 4 and 0.
+ * meaningful in `out`; split_k, group_m, wave_slots and partial_sums are launch-time parameters,
+ * returned as 1, 4, 0 and 0.
  */
 int rocm_sgemm_family_size(void);
 int rocm_sgemm_family_entry(int index, rocm_sgemm_config* out);

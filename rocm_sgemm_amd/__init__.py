@@ -53,12 +53,13 @@ class Config(ctypes.Structure):
     """struct rocm_sgemm_config."""
     _fields_ = [(n, ctypes.c_int) for n in
                 ("macro_m", "macro_n", "k_tile", "waves_m", "waves_n", "mfma", "stages", "split_k",
-                 "group_m", "wave_slots", "waves_k")]
+                 "group_m", "wave_slots", "waves_k", "partial_sums")]
 
     def as_dict(self):
         return {n: getattr(self, n) for n, _ in self._fields_}
 
-    _DEFAULTS = {"mfma": 32, "stages": 0, "split_k": 1, "group_m": 4, "wave_slots": 0, "waves_k": 1}
+    _DEFAULTS = {"mfma": 32, "stages": 0, "split_k": 1, "group_m": 4, "wave_slots": 0, "waves_k": 1,
+                 "partial_sums": 0}
 
     @classmethod
     def from_dict(cls, d):

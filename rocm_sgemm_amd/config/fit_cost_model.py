@@ -6,7 +6,7 @@ by a small analytic model of a launch's duration.  Its structure is fixed (see `
 restates the C++ `predict_us` of csrc/planner.cpp term by term); its constants are fitted here.
 
 Input: logs of `tuner --sweep M N K a b c --splits 1,2,4,8 --groups 4` (one line per timed config:
-`cfg <11 ints> avg_ms .. min_ms .. tflops .. ok 1`), one file per problem, named
+`cfg <12 ints> avg_ms .. min_ms .. tflops .. ok 1`), one file per problem, named
 `sweep_<M>_<N>_<K>*.log`.  `--collect DIR` writes them: it runs the tuner binary (on a GPU) on
 every problem of fit_problems.txt, the list the compiled constants were fitted on.  The fit minimises the squared error of log(time), weighting each config
 by exp(-(t / t_best - 1) / 0.25) so that the ordering among a problem's fast configs matters most.
@@ -25,7 +25,7 @@ import sys
 import numpy as np
 
 # (sweeps written before the waves_k field existed have ten integers per line)
-LINE = re.compile(r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+)(?: (\d+))? avg_ms ([\d.]+) "
+LINE = re.compile(r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+)(?: (\d+))?(?: \d+)? avg_ms ([\d.]+) "
                   r"min_ms ([\d.]+) tflops ([\d.]+) ok ([01])")
 KEYS = ["macro_m", "macro_n", "k_tile", "waves_m", "waves_n", "mfma", "stages", "split_k", "group_m",
         "wave_slots", "waves_k"]

@@ -17,6 +17,8 @@ describe a wave32 VALU kernel (thread tiles, threads_n); an MFMA kernel is descr
                         every K-tile over the whole wave tile and the partial tiles are summed
                         through LDS (1 = none); block size = 64 * waves_m * waves_n * waves_k
     split_k, group_m    launch-time only: K slices and tile-order band height
+    partial_sums        launch-time only: who adds up the partial tiles of a K split or a stream-K
+                        tail: 0 = the library decides, 1 = a second kernel, 2 = the GEMM launch
     wave_slots          launch-time only: 0 = deal the K range of a short last wave of tiles out
                         to all CUs (stream-K tail; slots asked from the runtime), 1 = never
 
@@ -42,22 +44,24 @@ PARAM_SPACE = {
     "group_m": [1, 2, 4, 8, 16],
     "wave_slots": [0, 1],
     "waves_k": [1, 2, 4],
+    "partial_sums": [0, 1, 2],
 }
 
 # A tile shape (what is compiled) is the tuple of SHAPE_KEYS; a config adds the launch-time
 # parameters.  CONFIG_KEYS is the field order of struct rocm_sgemm_config, of the tuner binary's
-# command line and of its `cfg` lines: waves_k, the youngest field, sits at the end of it.
+# command line and of its `cfg` lines: fields are appended as they are added, so waves_k sits
+# behind the first three launch-time parameters and partial_sums behind it.
 SHAPE_KEYS = ("macro_m", "macro_n", "k_tile", "waves_m", "waves_n", "mfma", "stages", "waves_k")
-CONFIG_KEYS = SHAPE_KEYS[:7] + ("split_k", "group_m", "wave_slots", "waves_k")
+CONFIG_KEYS = SHAPE_KEYS[:7] + ("split_k", "group_m", "wave_slots", "waves_k", "partial_sums")
 LAYOUTS = ("row_major", "col_major")
 
 
 def lds_bytes(macro_m, macro_n, k_tile, x_kc, y_kc, stages=0, waves_k=1):
     """LDS footprint; mirrors tile_config::LDS_BYTES in csrc/sgemm_mfma_kernel.hpp: padded images
     in two stages when register-staged, unpadded images in `stages` stages when direct-to-LDS;
-    with waves along K, at least the waves_k partial-tile images (rows padded by 8 floats)."""
+    with waves along K, at least the waves_k partial-tile images."""
     if stages >= 2:
-        exchange = waves_k * macro_m * (macro_n + 8) * 4 if waves_k > 1 else 0
+        exchange = waves_k * macro_m * macro_n * 4 if waves_k > 1 else 0
         return max(stages * (macro_m + macro_n) * k_tile * 4, exchange)
     x = macro_m * (k_tile + 4) if x_kc else k_tile * (macro_m + 4)
     y = macro_n * (k_tile + 4) if y_kc else k_tile * (macro_n + 4)
@@ -227,4 +231,5 @@ DEFAULT_CONFIG = {
     "group_m": 4,
     "wave_slots": 0,
     "waves_k": 1,
+    "partial_sums": 0,
 }

@@ -13,7 +13,9 @@ What differs, because the kernels do:
   * the space is small enough (tens of shapes x a few launch parameters) to be searched
     exhaustively in two phases, so no Optuna/TPE sampler is needed (Optuna is also not part of
     this environment): phase 1 sweeps all shapes at group_m = 4 with the split_k values that bring
-    the grid to at least one workgroup per CU, phase 2 re-times the best shapes over every group_m.
+    the grid to at least one workgroup per CU, phase 2 re-times the best shapes over every group_m,
+    phases 3 and 4 try the best configs without the stream-K tail and with the partial tiles summed
+    inside the launch / by a second kernel.
     `--budget` caps the number of trials per (size, layout) as in the reference.
 
 usage examples
@@ -36,7 +38,7 @@ import space  # noqa: E402
 
 LAYOUT_ALIASES = {"r": 0, "row_major": 0, "c": 1, "col_major": 1}
 SWEEP_LINE = re.compile(
-    r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) avg_ms ([\d.]+) min_ms ([\d.]+) "
+    r"cfg (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) (\d+) avg_ms ([\d.]+) min_ms ([\d.]+) "
     r"tflops ([\d.]+) ok ([01])")
 
 
@@ -178,6 +180,24 @@ class Tuner:
             cfg = dict(best["config"], wave_slots=1)
             if tuple(cfg.values()) not in seen:
                 ms = self.single(M, N, K, layout, cfg)
+                if ms is not None:
+                    trials.append({"config": cfg, "avg_ms": ms, "min_ms": ms, "tflops": 0.0,
+                                   "ok": True})
+        # phase 4: the best few configs that leave partial tiles (K split or stream-K tail) with the
+        # summation forced into the GEMM launch and forced into a second kernel
+        trials.sort(key=lambda t: t["avg_ms"])
+        for t in list(trials[:3]):
+            if t["config"]["split_k"] == 1 and t["config"]["wave_slots"] == 1:
+                continue
+            for sums in (1, 2):
+                if left <= 0:
+                    break
+                cfg = dict(t["config"], partial_sums=sums)
+                if tuple(cfg.values()) in seen:
+                    continue
+                seen.add(tuple(cfg.values()))
+                ms = self.single(M, N, K, layout, cfg)
+                left -= 1
                 if ms is not None:
                     trials.append({"config": cfg, "avg_ms": ms, "min_ms": ms, "tflops": 0.0,
                                    "ok": True})

@@ -4,10 +4,10 @@
 // a trial is a plain library call - rocm_sgemm_f32_with_config - because every tile shape of the
 // search space is compiled into librocm_sgemm; nothing is compiled at run time.
 //
-//   tuner M N K macro_m macro_n k_tile waves_m waves_n mfma stages split_k group_m wave_slots waves_k A B C [iters] [warmup]
+//   tuner M N K macro_m macro_n k_tile waves_m waves_n mfma stages split_k group_m wave_slots waves_k partial_sums A B C [iters] [warmup]
 //       layouts: 0 = row_major, 1 = col_major.  Prints "time: <avg> ms  min: <min> ms ...".
-//   tuner --sweep M N K A B C [--iters n] [--warmup n] [--splits a,b,..] [--groups a,b,..] [--slots a,b,..]
-//       one line per (tile shape, split_k, group_m):  "cfg <11 ints> avg_ms <..> min_ms <..> tflops <..> ok <0|1>"
+//   tuner --sweep M N K A B C [--iters n] [--warmup n] [--splits a,b,..] [--groups a,b,..] [--slots a,b,..] [--sums a,b]
+//       one line per (tile shape, split_k, group_m, ..):  "cfg <12 ints> avg_ms <..> min_ms <..> tflops <..> ok <0|1>"
 //
 // Inputs are uniform[-1, 1) from a fixed xorshift stream; every trial is checked on 256 sampled
 // entries against an fp64 dot product so that a mis-tuned config can never enter the table.
@@ -186,9 +186,9 @@ int usage()
 {
     std::fprintf(stderr,
                  "usage: tuner M N K macro_m macro_n k_tile waves_m waves_n mfma stages split_k group_m "
-                 "wave_slots waves_k A B C [iters] [warmup]\n"
+                 "wave_slots waves_k partial_sums A B C [iters] [warmup]\n"
                  "       tuner --sweep M N K A B C [--iters n] [--warmup n] [--splits a,b] "
-                 "[--groups a,b]\n");
+                 "[--groups a,b] [--slots a,b] [--sums a,b]\n");
     return 2;
 }
 
@@ -204,7 +204,7 @@ int main(int argc, char** argv)
         p.K = std::strtoull(argv[4], nullptr, 10);
         p.la = std::atoi(argv[5]), p.lb = std::atoi(argv[6]), p.lc = std::atoi(argv[7]);
         int              iters = 10, warmup = 2;
-        std::vector<int> splits{1}, groups{4}, slots{0};
+        std::vector<int> splits{1}, groups{4}, slots{0}, sums{0};
         for(int i = 8; i + 1 < argc; i += 2)
         {
             if(!std::strcmp(argv[i], "--iters")) iters = std::atoi(argv[i + 1]);
@@ -212,6 +212,7 @@ int main(int argc, char** argv)
             else if(!std::strcmp(argv[i], "--splits")) splits = parse_list(argv[i + 1]);
             else if(!std::strcmp(argv[i], "--groups")) groups = parse_list(argv[i + 1]);
             else if(!std::strcmp(argv[i], "--slots")) slots = parse_list(argv[i + 1]);
+            else if(!std::strcmp(argv[i], "--sums")) sums = parse_list(argv[i + 1]);
             else return usage();
         }
         setup(p);
@@ -228,17 +229,21 @@ int main(int argc, char** argv)
                 if(s > 1 && (static_cast<size_t>(s) * cfg.k_tile * 2 > p.K || tiles * s > 2048)) continue;
                 for(int g : groups)
                 for(int w : slots)
+                for(int u : sums)
                 {
                     if(w != 0 && s > 1) continue; // the tail split only applies without split_k
-                    cfg.split_k    = s;
-                    cfg.group_m    = g;
-                    cfg.wave_slots = w;
+                    if(u != sums.front() && s == 1 && w == 1) continue; // no partial tiles to add up
+                    cfg.split_k      = s;
+                    cfg.group_m      = g;
+                    cfg.wave_slots   = w;
+                    cfg.partial_sums = u;
                     if(!rocm_sgemm_config_supported(&cfg, p.lc, p.la, p.lb)) continue;
                     const timing t = run_trial(p, cfg, iters, warmup);
                     if(!t.launched) continue;
-                    std::printf("cfg %d %d %d %d %d %d %d %d %d %d %d avg_ms %.4f min_ms %.4f tflops %.2f ok %d\n",
+                    std::printf("cfg %d %d %d %d %d %d %d %d %d %d %d %d avg_ms %.4f min_ms %.4f tflops %.2f ok %d\n",
                                 cfg.macro_m, cfg.macro_n, cfg.k_tile, cfg.waves_m, cfg.waves_n,
-                                cfg.mfma, cfg.stages, cfg.split_k, cfg.group_m, cfg.wave_slots, cfg.waves_k, t.avg_ms,
+                                cfg.mfma, cfg.stages, cfg.split_k, cfg.group_m, cfg.wave_slots, cfg.waves_k,
+                                cfg.partial_sums, t.avg_ms,
                                 t.min_ms,
                                 flops / (t.avg_ms * 1e-3) * 1e-12, t.correct ? 1 : 0);
                     std::fflush(stdout);
@@ -249,7 +254,7 @@ int main(int argc, char** argv)
         return 0;
     }
 
-    if(argc < 18)
+    if(argc < 19)
     {
         return usage();
     }
@@ -260,10 +265,10 @@ int main(int argc, char** argv)
     rocm_sgemm_config cfg{std::atoi(argv[4]), std::atoi(argv[5]), std::atoi(argv[6]),
                           std::atoi(argv[7]), std::atoi(argv[8]), std::atoi(argv[9]),
                           std::atoi(argv[10]), std::atoi(argv[11]), std::atoi(argv[12]),
-                          std::atoi(argv[13]), std::atoi(argv[14])};
-    p.la = std::atoi(argv[15]), p.lb = std::atoi(argv[16]), p.lc = std::atoi(argv[17]);
-    const int iters  = argc > 18 ? std::atoi(argv[18]) : 20;
-    const int warmup = argc > 19 ? std::atoi(argv[19]) : 3;
+                          std::atoi(argv[13]), std::atoi(argv[14]), std::atoi(argv[15])};
+    p.la = std::atoi(argv[16]), p.lb = std::atoi(argv[17]), p.lc = std::atoi(argv[18]);
+    const int iters  = argc > 19 ? std::atoi(argv[19]) : 20;
+    const int warmup = argc > 20 ? std::atoi(argv[20]) : 3;
     if(!rocm_sgemm_config_supported(&cfg, p.lc, p.la, p.lb))
     {
         std::fprintf(stderr, "unsupported config: %s\n", rocm_sgemm_last_error());

@@ -119,6 +119,11 @@ struct workspace_buffer
     void*      ptr   = nullptr;
     size_t     bytes = 0;
 };
+// Every workspace starts with the counters of the launches that sum their partial tiles
+// themselves (kernel::gemm_args::counters): always at the same place, zero when the buffer is
+// created and left at zero by every launch that uses them.  The partial tiles follow.
+constexpr size_t counter_slots = 16384;
+constexpr size_t counter_bytes = counter_slots * sizeof(unsigned);
 std::mutex                                workspace_table_lock;
 std::map<workspace_key, workspace_buffer> workspaces;
 
@@ -165,6 +170,14 @@ hipError_t workspace_get(void** ptr, size_t bytes, hipStream_t stream, bool* str
     }
     const size_t want = bytes + bytes / 4; // head room: slightly larger problems do not regrow
     err               = hipMalloc(&buf->ptr, want);
+    if(err == hipSuccess)
+    {
+        err = hipMemset(buf->ptr, 0, counter_bytes < want ? counter_bytes : want); // the counters start at zero
+        if(err != hipSuccess)
+        {
+            (void)hipFree(buf->ptr);
+        }
+    }
     if(err != hipSuccess)
     {
         buf->ptr = nullptr;
@@ -180,8 +193,10 @@ hipError_t workspace_get(void** ptr, size_t bytes, hipStream_t stream, bool* str
 // own copy at its own address).  On the host the array's name is only a handle for
 // hipGetSymbolAddress, not a device address; the address is looked up once per device, with that
 // device current, and only that pointer is ever handed to a kernel.
+// It is laid out like an allocated workspace: the counters (zero from the start, like all of the
+// array), then ROCM_SGEMM_NO_ALLOC_SCRATCH_BYTES for partial tiles.
 constexpr size_t scratch_floats = ROCM_SGEMM_NO_ALLOC_SCRATCH_BYTES / sizeof(float);
-static __device__ __align__(256) float scratch[scratch_floats];
+static __device__ __align__(256) float scratch[counter_bytes / sizeof(float) + scratch_floats];
 
 constexpr int       scratch_max_devices = 64;
 std::atomic<float*> scratch_address[scratch_max_devices];
@@ -267,9 +282,10 @@ bool config_supported(const rocm_sgemm_config& c, int layout_c, int layout_a, in
         error = "layout must be ROCM_SGEMM_ROW_MAJOR (0) or ROCM_SGEMM_COL_MAJOR (1)";
         return false;
     }
-    if(c.split_k < 1 || c.split_k > 1024 || c.group_m < 1 || c.wave_slots < 0)
+    if(c.split_k < 1 || c.split_k > 1024 || c.group_m < 1 || c.wave_slots < 0 || c.partial_sums < 0
+       || c.partial_sums > 2)
     {
-        error = "split_k must be in [1, 1024], group_m >= 1 and wave_slots >= 0";
+        error = "split_k must be in [1, 1024], group_m >= 1, wave_slots >= 0 and partial_sums 0, 1 or 2";
         return false;
     }
     const bool swap = layout_c == ROCM_SGEMM_COL_MAJOR;
@@ -325,9 +341,10 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
         error = "layout must be ROCM_SGEMM_ROW_MAJOR (0) or ROCM_SGEMM_COL_MAJOR (1)";
         return ROCM_SGEMM_STATUS_INVALID_ARG;
     }
-    if(c.split_k < 1 || c.split_k > 1024 || c.group_m < 1 || c.wave_slots < 0)
+    if(c.split_k < 1 || c.split_k > 1024 || c.group_m < 1 || c.wave_slots < 0 || c.partial_sums < 0
+       || c.partial_sums > 2)
     {
-        error = "split_k must be in [1, 1024], group_m >= 1 and wave_slots >= 0";
+        error = "split_k must be in [1, 1024], group_m >= 1, wave_slots >= 0 and partial_sums 0, 1 or 2";
         return ROCM_SGEMM_STATUS_BAD_CONFIG;
     }
     if(p.batch < 1 || p.batch > 65535)
@@ -516,6 +533,30 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     {
         workspace_floats = static_cast<size_t>(args.tail_groups) * 2 * bm * bn;
     }
+    // Who adds the partial tiles up: the launch itself (the wave that completes a tile's counter,
+    // see kernel::gemm_args::counters) or a second kernel.  The first saves a launch and the
+    // write-back of the partial tiles at the end of the GEMM kernel, and the summing of one tile
+    // overlaps with the multiplication of others: 2 to 10 % on products of 80 us and more.  But
+    // every wave waits for its stores and its ticket, and the wave that adds up reads all parts of
+    // its share one after the other: on products of 20 to 45 us, where all tiles finish together
+    // and nothing overlaps, it costs 2 to 5 us more than the second launch.  And one wave reads at
+    // a few GB/s, so its share must be little data.  Hence, unless the config says otherwise:
+    // in the launch for products of at least 8 GFLOP whose waves have at most 48 KB to add up.
+    // (Possible at all only with at most four waves that own at most a 64 x 64 share of the tile
+    // each, kernel::tile_config::SUMS_IN_LAUNCH, 32-bit byte offsets into a partial matrix, and
+    // counters for every (batch, tile, wave).)
+    const int    waves_per_group = wm * wn * (c.waves_k > 1 ? c.waves_k : 1);
+    const size_t counters_needed
+        = static_cast<size_t>(p.batch) * static_cast<size_t>(args.tail_groups > 0 ? tail_tiles : tiles) * waves_per_group;
+    const long long parts          = args.tail_groups > 0 ? (k_tiles + args.tail_per - 1) / args.tail_per + 1 : split;
+    const long long bytes_per_wave = parts * bm * bn * 4ll / waves_per_group;
+    const double    flop           = 2.0 * static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K)
+                        * static_cast<double>(p.batch);
+    const bool      possible = !scaled && (split > 1 || args.tail_groups > 0) && counters_needed <= counter_slots
+                          && bm * bn / waves_per_group <= 64 * 64 && waves_per_group <= 4 && count < (1ull << 29);
+    bool in_launch = possible
+                     && (c.partial_sums == 2 || (c.partial_sums == 0 && flop >= 8.0e9 && bytes_per_wave <= 48 * 1024));
+    void* workspace_base = nullptr;
     if(workspace_floats > 0 && p.no_alloc)
     {
         // the fixed scratch array of this GPU: nothing is allocated, every call on the GPU shares it
@@ -534,20 +575,27 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
             error = std::string("address of the scratch array not available: ") + hipGetErrorString(err);
             return ROCM_SGEMM_STATUS_LAUNCH_FAILED;
         }
-        args.partial = ws;
+        workspace_base = ws;
     }
     else if(workspace_floats > 0)
     {
         // the library's buffer of this stream (see workspace_get)
         void*      ws  = nullptr;
-        hipError_t err = workspace_get(&ws, workspace_floats * sizeof(float), stream, &workspace_stream_ordered,
-                                       workspace_guard);
+        hipError_t err = workspace_get(&ws, counter_bytes + workspace_floats * sizeof(float), stream,
+                                       &workspace_stream_ordered, workspace_guard);
         if(err != hipSuccess)
         {
             error = std::string("workspace allocation failed: ") + hipGetErrorString(err);
             return ROCM_SGEMM_STATUS_LAUNCH_FAILED;
         }
-        args.partial = static_cast<float*>(ws);
+        workspace_base = ws;
+        // a one-off allocation (stream capture) comes with counters that nobody has cleared
+        in_launch = in_launch && !workspace_stream_ordered;
+    }
+    if(workspace_base != nullptr)
+    {
+        args.partial  = reinterpret_cast<float*>(static_cast<char*>(workspace_base) + counter_bytes);
+        args.counters = in_launch ? static_cast<unsigned*>(workspace_base) : nullptr;
     }
     const int       ldc_out    = args.ldp;
     const long long stride_out = args.stride_p;
@@ -561,7 +609,11 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
 
     const kernel::output_scale scale{p.alpha, p.beta};
     hipError_t err = fn(args, static_cast<unsigned>(groups), batches, stream);
-    if(err == hipSuccess && (split > 1 || scaled))
+    if(args.counters != nullptr)
+    {
+        // the launch has summed its partial tiles itself
+    }
+    else if(err == hipSuccess && (split > 1 || scaled))
     {
         const bool vec4 = args.cols % 4 == 0 && ldc_out % 4 == 0 && aligned16(p.C)
                           && (batches == 1 || stride_out % 4 == 0);
@@ -587,7 +639,7 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     }
     if(workspace_stream_ordered)
     {
-        const hipError_t ferr = hipFreeAsync(args.partial, stream);
+        const hipError_t ferr = hipFreeAsync(workspace_base, stream);
         if(err == hipSuccess)
         {
             err = ferr;

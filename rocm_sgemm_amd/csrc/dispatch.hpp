@@ -38,7 +38,7 @@ const rocm_sgemm_config& select_config(const tuned_entry*       table,
 /// Config the library runs for `batch` products of one shape: a single product that is itself a
 /// table entry gets its entry; anything else the cheapest, by the cost model below, of the
 /// nearest entry's config (K split fitted to the problem's own tile count), those of the next
-/// three nearest entries and the larger direct-to-LDS shapes of the family at split_k 1, 2, 4, 8 -
+/// three nearest entries and the larger direct-to-LDS shapes of the family at split_k 1, 2, 3, 4, 6, 8 -
 /// the nearest entry's config stays unless another is predicted at least 4 % faster.
 rocm_sgemm_config plan_config(size_t m, size_t n, size_t k, int layout_a, int layout_b, int layout_c,
                               size_t batch = 1);

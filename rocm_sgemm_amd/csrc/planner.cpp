@@ -316,7 +316,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     // prices the configs of the four nearest entries of the same layouts and kind, and every
     // direct-to-LDS tile shape of the family with 32 x 32 MFMAs and tiles of at least 64 x 64 (or
     // smaller ones with waves along K, which keep a large wave tile) at
-    // split_k 1, 2, 4 and 8; the cheapest of them replaces the nearest entry's config only if
+    // split_k 1, 2, 3, 4, 6 and 8; the cheapest of them replaces the nearest entry's config only if
     // the model expects it to be at least 4 % faster (about the model's own error).
     const auto aligned_kind = [](size_t a, size_t b, size_t c) { return a % 4 == 0 && b % 4 == 0 && c % 4 == 0; };
     constexpr int   max_candidates = 4;
@@ -371,7 +371,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
         family_entry(i, &s);
         if(s.stages < 2 || s.mfma != 32 || ((s.macro_m < 64 || s.macro_n < 64) && s.waves_k <= 1)) continue;
         const long long k_tiles = static_cast<long long>((k + s.k_tile - 1) / s.k_tile);
-        for(int split = 1; split <= 8; split *= 2)
+        for(const int split : {1, 2, 3, 4, 6, 8})
         {
             if(split > 1 && k_tiles < 2LL * split) break; // at least two K-tiles per slice
             consider(rocm_sgemm_config{s.macro_m, s.macro_n, s.k_tile, s.waves_m, s.waves_n, s.mfma, s.stages,

@@ -105,6 +105,11 @@ struct gemm_args
     int tail_begin; // == grid_m * grid_n when there is no tail
     int tail_groups; // 0 = none
     int tail_per;
+    // Partial tiles summed inside this launch (split_k > 1 or a stream-K tail): one counter per
+    // (batch, tile, wave of the workgroup), all zero when the launch starts and zero again when it
+    // ends; the wave that completes a counter adds up the tile's parts and stores the result.
+    // Null: the partial tiles are left for a second kernel.
+    unsigned* counters;
 };
 
 template<int BM_, int BN_, int BK_, int WM_, int WN_, int MI_, bool X_KC_, bool Y_KC_, bool EDGE_, int NS_ = 0,
@@ -141,6 +146,11 @@ struct tile_config
     static constexpr int KB  = 4 * (64 / MI); // depth of a k-block: 4 MFMA steps
     static constexpr int NKB = BK / KB; // k-blocks per K-tile
     static constexpr int NKBW = NKB / WK; // k-blocks of a K-tile one wave multiplies
+    // Whether the kernel can add up the partial tiles of a K split or a stream-K tail itself
+    // (gemm_args::counters): a wave's share of the macro tile is at most 64 x 64, and the workgroup
+    // has at most four waves (with eight, two waves share a SIMD's registers and the summing code
+    // does not fit beside the accumulators).
+    static constexpr bool SUMS_IN_LAUNCH = BM * BN / (WM * WN * WK) <= 64 * 64 && WM * WN * WK <= 4;
 
     // Interleave width of a row-contiguous operand (tiles fed by one LDS read).
     static constexpr int VM = TM >= 4 ? 4 : TM;
@@ -160,11 +170,13 @@ struct tile_config
     static constexpr int Y_SIZE = Y_KC ? BN * LDY : BK * LDY;
     static constexpr int STAGE  = X_SIZE + Y_SIZE;
     static constexpr int STAGES = DTL ? NS : 2;
-    // WK > 1: after the main loop every wave-grid replica leaves its partial tile in LDS as a
-    // BM x BN row-major image with rows EX_LD floats apart (the 8 floats of padding put the two
-    // rows a 32 x 32 MFMA tile's lane groups write at once 32 banks apart).
-    static constexpr int EX_LD     = BN + 8;
-    static constexpr int EX_FLOATS = WK > 1 ? WK * BM * EX_LD : 0;
+    // WK > 1: after the main loop every wave-grid replica leaves its partial tile in LDS as an
+    // unpadded BM x BN row-major image, which the workgroup then reads linearly (thread t the
+    // t-th group of four floats: conflict-free).  The two lane groups of an MFMA tile write rows
+    // that differ in bit EX_ROW_BIT and would hit the same banks; so bit 5 of an element's linear
+    // index (32 floats = half of the 64 banks) is flipped where that row bit is set.
+    static constexpr int EX_ROW_BIT = X_KC ? 2 : (VM == 4 ? 4 : (VM == 2 ? 3 : 2));
+    static constexpr int EX_FLOATS  = WK > 1 ? WK * BM * BN : 0;
     static constexpr int LDS_FLOATS = STAGES * STAGE > EX_FLOATS ? STAGES * STAGE : EX_FLOATS;
     static constexpr int LDS_BYTES = LDS_FLOATS * 4;
 
@@ -923,130 +935,75 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
 #if defined(__HIP_DEVICE_COMPILE__)
     asm volatile("" : "+v"(h_e), "+v"(c_e));
 #endif
-    float* __restrict__ P;
-    int ldp, row_base, col_base, row_end, col_end;
-    if(tail)
+    // Where a tile goes or comes from: base, row stride, origin of the macro tile, matrix extent.
+    struct tile_place
     {
-        P   = args.partial + (static_cast<size_t>(tail_g) * 2 + seg) * (BM * BN);
-        ldp = BN, row_base = 0, col_base = 0, row_end = BM, col_end = BN;
-    }
-    else if(args.split_k > 1)
-    {
-        P = args.partial
-            + (static_cast<size_t>(batch) * args.split_k + slice) * args.rows * static_cast<size_t>(args.cols);
-        ldp = args.cols, row_base = m0, col_base = n0, row_end = args.rows, col_end = args.cols;
-    }
-    else
-    {
-        P   = args.P + batch * args.stride_p;
-        ldp = args.ldp, row_base = m0, col_base = n0, row_end = args.rows, col_end = args.cols;
-    }
-    if constexpr(WK > 1)
-    {
-        // Waves along K: every replica of the wave grid holds a partial of the whole macro tile.
-        // Each leaves it in LDS as a row-major BM x BN image; then the workgroup sums the images in
-        // replica order (fixed, so the result does not depend on timing) and stores whole rows,
-        // four adjacent columns per thread.
-        constexpr int EX_LD = Cfg::EX_LD;
-        __syncthreads(); // every wave is done with the stages: the images reuse their memory
-        float* image = lds + wk * (BM * EX_LD);
+        float* base;
+        int    ld, row0, col0, row_end, col_end;
+    };
+    const bool       to_partial = tail || args.split_k > 1;
+    const tile_place result{args.P + batch * args.stride_p, args.ldp, m0, n0, args.rows, args.cols};
+    // the partial of split-K slice s (tiles at their place in a packed rows x cols matrix)
+    auto slice_place = [&](int s) {
+        return tile_place{args.partial
+                              + (static_cast<size_t>(batch) * args.split_k + s) * args.rows * static_cast<size_t>(args.cols),
+                          args.cols, m0, n0, args.rows, args.cols};
+    };
+    // the partial tile of segment s of tail workgroup g (never clipped)
+    auto segment_place = [&](int g, int s) {
+        return tile_place{args.partial + (static_cast<size_t>(g) * 2 + s) * (BM * BN), BN, 0, 0, BM, BN};
+    };
+    const tile_place mine = tail ? segment_place(tail_g, seg) : (args.split_k > 1 ? slice_place(slice) : result);
+
+    // Plain stores of one row of MFMA tiles: `vals[j][v]` is accumulator register v of tile (i, j),
+    // v in [v_begin, v_begin + v_count); 128-bit where the lane's values are adjacent.
+    auto put_row = [&](const tile_place& t, int i, auto& vals, auto v_begin_c, auto v_count_c) {
 #pragma unroll
-        for(int i = 0; i < TM; ++i)
-#pragma unroll
-            for(int v = 0; v < ACC; ++v)
-            {
-                const int r = wm0 + impl::tile_index<X_KC, VM, MI>(i, impl::acc_row<MI>(v, h_e));
-#pragma unroll
-                for(int j = 0; j < TN; ++j)
-                    image[r * EX_LD + wn0 + impl::tile_index<Y_KC, VN, MI>(j, c_e)] = acc[i][j][v];
-            }
-        __syncthreads();
-#pragma unroll
-        for(int g = 0; g < BM * BN / 4 / NT; ++g)
-        {
-            const int q = g * NT + tid;
-            const int r = q / (BN / 4);
-            const int n = (q % (BN / 4)) * 4;
-            f32x4     o = *reinterpret_cast<const f32x4*>(lds + r * EX_LD + n);
-#pragma unroll
-            for(int w = 1; w < WK; ++w)
-                o += *reinterpret_cast<const f32x4*>(lds + w * (BM * EX_LD) + r * EX_LD + n);
-            const int row = row_base + r;
-            const int col = col_base + n;
-            float*    dst = P + static_cast<size_t>(row) * ldp + col;
-            if constexpr(!EDGE)
-            {
-                *reinterpret_cast<f32x4*>(dst) = o;
-            }
-            else if(row < row_end)
-            {
-                if(col + 3 < col_end)
-                {
-                    *reinterpret_cast<f32x4_e*>(dst) = o;
-                }
-                else
-                {
-                    if(col < col_end) dst[0] = o.x;
-                    if(col + 1 < col_end) dst[1] = o.y;
-                    if(col + 2 < col_end) dst[2] = o.z;
-                }
-            }
-        }
-    }
-    else
-    {
-#pragma unroll
-    for(int i = 0; i < TM; ++i)
-    {
-#pragma unroll
-        for(int v = 0; v < ACC; ++v)
+        for(int v = decltype(v_begin_c)::value; v < decltype(v_begin_c)::value + decltype(v_count_c)::value; ++v)
         {
             const int mi  = impl::acc_row<MI>(v, h_e);
-            const int row = row_base + wm0 + impl::tile_index<X_KC, VM, MI>(i, mi);
-            if(EDGE && row >= row_end)
+            const int row = t.row0 + wm0 + impl::tile_index<X_KC, VM, MI>(i, mi);
+            if(EDGE && row >= t.row_end)
             {
                 continue;
             }
-            float* prow = P + static_cast<size_t>(row) * ldp;
+            float* prow = t.base + static_cast<size_t>(row) * t.ld;
             if constexpr(!Y_KC && VN > 1)
             {
 #pragma unroll
                 for(int g = 0; g < TN / VN; ++g)
                 {
-                    const int col = col_base + wn0 + g * MI * VN + VN * c_e;
+                    const int col = t.col0 + wn0 + g * MI * VN + VN * c_e;
                     if constexpr(VN == 4)
                     {
-                        const f32x4 o = {acc[i][g * 4 + 0][v],
-                                         acc[i][g * 4 + 1][v],
-                                         acc[i][g * 4 + 2][v],
-                                         acc[i][g * 4 + 3][v]};
+                        const f32x4 o = {vals[g * 4 + 0][v], vals[g * 4 + 1][v], vals[g * 4 + 2][v], vals[g * 4 + 3][v]};
                         if constexpr(!EDGE)
                         {
                             *reinterpret_cast<f32x4*>(prow + col) = o;
                         }
-                        else if(col + 3 < col_end)
+                        else if(col + 3 < t.col_end)
                         {
                             *reinterpret_cast<f32x4_e*>(prow + col) = o;
                         }
                         else
                         {
-                            if(col < col_end) prow[col] = o.x;
-                            if(col + 1 < col_end) prow[col + 1] = o.y;
-                            if(col + 2 < col_end) prow[col + 2] = o.z;
+                            if(col < t.col_end) prow[col] = o.x;
+                            if(col + 1 < t.col_end) prow[col + 1] = o.y;
+                            if(col + 2 < t.col_end) prow[col + 2] = o.z;
                         }
                     }
                     else
                     {
-                        const f32x2 o = {acc[i][g * 2 + 0][v], acc[i][g * 2 + 1][v]};
+                        const f32x2 o = {vals[g * 2 + 0][v], vals[g * 2 + 1][v]};
                         if constexpr(!EDGE)
                         {
                             *reinterpret_cast<f32x2*>(prow + col) = o;
                         }
-                        else if(col + 1 < col_end)
+                        else if(col + 1 < t.col_end)
                         {
                             *reinterpret_cast<f32x2_e*>(prow + col) = o;
                         }
-                        else if(col < col_end)
+                        else if(col < t.col_end)
                         {
                             prow[col] = o.x;
                         }
@@ -1058,16 +1015,279 @@ __global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args arg
 #pragma unroll
                 for(int j = 0; j < TN; ++j)
                 {
-                    const int col = col_base + wn0 + impl::tile_index<Y_KC, VN, MI>(j, c_e);
-                    if(!EDGE || col < col_end)
+                    const int col = t.col0 + wn0 + impl::tile_index<Y_KC, VN, MI>(j, c_e);
+                    if(!EDGE || col < t.col_end)
                     {
-                        prow[col] = acc[i][j][v];
+                        prow[col] = vals[j][v];
                     }
                 }
             }
         }
+    };
+
+    // Traffic between workgroups of one launch (the parts of a tile that is summed in the launch):
+    //   SHARE    stores other workgroups' waves will read: written through to memory, never left
+    //            dirty in this XCD's L2
+    //   FETCH    value  = what another workgroup shared: never a line a cache still holds from before
+    //   GATHER   value += the same
+    // These are buffer accesses with the agent-scope cache policy (the bits agent-scope atomic loads
+    // and stores carry): one 32-bit offset per element from a wave-uniform base, elements outside
+    // the matrix get an offset the range check rejects (their stores are dropped, their loads
+    // return zero), so the code has no branches.  Offsets stay below 2 GiB (the host checks).
+    constexpr int SHARE = 1, FETCH = 2, GATHER = 3;
+    constexpr int agent_scope = 16; // cache policy bit sc1
+    auto coherent = [](auto mode_c, __amdgpu_buffer_rsrc_t rsrc, int byte_offset, float value) -> float {
+        constexpr int mode = decltype(mode_c)::value;
+#if defined(__HIP_DEVICE_COMPILE__)
+        if constexpr(mode == SHARE)
+        {
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), rsrc, byte_offset, 0, agent_scope);
+            return value;
+        }
+        else
+        {
+            const float got = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, agent_scope));
+            return mode == FETCH ? got : value + got;
+        }
+#else
+        (void)rsrc, (void)byte_offset;
+        return value;
+#endif
+    };
+    auto descriptor = [](const tile_place& t) {
+        return __builtin_amdgcn_make_buffer_rsrc(t.base, 0, 0x7FFFFFFF, 0x00020000);
+    };
+    constexpr int rejected = static_cast<int>(0x80000000u); // beyond any buffer declared above
+    auto coherent_row = [&](auto mode_c, const tile_place& t, int i, auto& vals, auto v_begin_c, auto v_count_c) {
+        constexpr int                mode = decltype(mode_c)::value;
+        const __amdgpu_buffer_rsrc_t rsrc = descriptor(t);
+#pragma unroll
+        for(int v = decltype(v_begin_c)::value; v < decltype(v_begin_c)::value + decltype(v_count_c)::value; ++v)
+        {
+            const int  row    = t.row0 + wm0 + impl::tile_index<X_KC, VM, MI>(i, impl::acc_row<MI>(v, h_e));
+            const bool row_ok = !EDGE || row < t.row_end;
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+            {
+                const int   col = t.col0 + wn0 + impl::tile_index<Y_KC, VN, MI>(j, c_e);
+                const int   off = row_ok && (!EDGE || col < t.col_end) ? (row * t.ld + col) * 4 : rejected;
+                const float got = coherent(mode_c, rsrc, off, vals[j][v]);
+                if constexpr(mode >= FETCH) vals[j][v] = got;
+            }
+#if defined(__HIP_DEVICE_COMPILE__)
+            // keeps the offsets of later rows from being computed (and held in registers) up front
+            __builtin_amdgcn_sched_barrier(0);
+#endif
+        }
+    };
+    // With waves along K the lane's share is `summed` instead: four adjacent columns of NSUM rows
+    // of the tile the workgroup has added up from the replicas' images.
+    constexpr int NSUM = WK > 1 ? BM * BN / 4 / NT : 1;
+    f32x4         summed[NSUM];
+    auto          put_summed = [&](const tile_place& t) {
+#pragma unroll
+        for(int g = 0; g < NSUM; ++g)
+        {
+            const int p   = (g * NT + tid) * 4; // where the image held the values (see EX_ROW_BIT)
+            const int l   = p ^ ((((p / BN) >> Cfg::EX_ROW_BIT) & 1) << 5);
+            const int row = t.row0 + l / BN;
+            const int col = t.col0 + l % BN;
+            float*    dst = t.base + static_cast<size_t>(row) * t.ld + col;
+            if constexpr(!EDGE)
+            {
+                *reinterpret_cast<f32x4*>(dst) = summed[g];
+            }
+            else if(row < t.row_end)
+            {
+                if(col + 3 < t.col_end)
+                {
+                    *reinterpret_cast<f32x4_e*>(dst) = summed[g];
+                }
+                else
+                {
+                    if(col < t.col_end) dst[0] = summed[g].x;
+                    if(col + 1 < t.col_end) dst[1] = summed[g].y;
+                    if(col + 2 < t.col_end) dst[2] = summed[g].z;
+                }
+            }
+        }
+    };
+    auto coherent_summed = [&](auto mode_c, const tile_place& t) {
+        constexpr int                mode = decltype(mode_c)::value;
+        const __amdgpu_buffer_rsrc_t rsrc = descriptor(t);
+#pragma unroll
+        for(int g = 0; g < NSUM; ++g)
+        {
+            const int  p      = (g * NT + tid) * 4; // where the image held the values (see EX_ROW_BIT)
+            const int  l      = p ^ ((((p / BN) >> Cfg::EX_ROW_BIT) & 1) << 5);
+            const int  row    = t.row0 + l / BN;
+            const int  col    = t.col0 + l % BN;
+            const bool row_ok = !EDGE || row < t.row_end;
+#pragma unroll
+            for(int e = 0; e < 4; ++e)
+            {
+                const int   off = row_ok && (!EDGE || col + e < t.col_end) ? (row * t.ld + col + e) * 4 : rejected;
+                const float got = coherent(mode_c, rsrc, off, summed[g][e]);
+                if constexpr(mode >= FETCH) summed[g][e] = got;
+            }
+        }
+    };
+    // The lane's whole share: plain stores, or stores for other workgroups to read.
+    auto put_tile = [&](const tile_place& t) {
+        if constexpr(WK > 1)
+            put_summed(t);
+        else
+            impl::static_for<0, TM>([&](auto i_c) {
+                put_row(t, decltype(i_c)::value, acc[decltype(i_c)::value], std::integral_constant<int, 0>{},
+                        std::integral_constant<int, ACC>{});
+            });
+    };
+    auto share_tile = [&](const tile_place& t) {
+        if constexpr(WK > 1)
+            coherent_summed(std::integral_constant<int, SHARE>{}, t);
+        else
+            impl::static_for<0, TM>([&](auto i_c) {
+                coherent_row(std::integral_constant<int, SHARE>{}, t, decltype(i_c)::value, acc[decltype(i_c)::value],
+                             std::integral_constant<int, 0>{}, std::integral_constant<int, ACC>{});
+            });
+    };
+    // The sum of the parts `place(n)`, n = 0 .. count - 1, added in that order, stored to the
+    // result.  The sums live in registers of their own: arithmetic on the accumulators would pull
+    // them out of the accumulation registers for the whole kernel.
+    auto sum_parts = [&](int count, auto&& place) {
+        if constexpr(WK > 1)
+        {
+            coherent_summed(std::integral_constant<int, FETCH>{}, place(0));
+            for(int n = 1; n < count; ++n)
+                coherent_summed(std::integral_constant<int, GATHER>{}, place(n));
+            put_summed(result);
+        }
+        else
+        {
+            // about 32 values of the lane at a time: enough loads in flight, few registers
+            constexpr int VCH = impl::max_int(1, (32 / TN < ACC ? 32 / TN : ACC));
+            impl::static_for<0, TM*(ACC / VCH)>([&](auto n_c) {
+                constexpr int                          i = decltype(n_c)::value / (ACC / VCH);
+                const std::integral_constant<int, (decltype(n_c)::value % (ACC / VCH)) * VCH> v0;
+                const std::integral_constant<int, VCH>                                         vn;
+                acc_t                                  sum[TN];
+                coherent_row(std::integral_constant<int, FETCH>{}, place(0), i, sum, v0, vn);
+                for(int n = 1; n < count; ++n)
+                    coherent_row(std::integral_constant<int, GATHER>{}, place(n), i, sum, v0, vn);
+                put_row(result, i, sum, v0, vn);
+            });
+        }
+    };
+
+    if constexpr(WK > 1)
+    {
+        // Waves along K: every replica of the wave grid holds a partial of the whole macro tile.
+        // Each leaves it in LDS as a row-major BM x BN image; then the workgroup sums the images in
+        // replica order (fixed, so the result does not depend on timing); a thread keeps four
+        // adjacent columns of NSUM rows.
+        // linear index of element (r, n) of an image, bank-swizzled (tile_config::EX_ROW_BIT)
+        auto image_index = [](int r, int n) { return (r * BN + n) ^ (((r >> Cfg::EX_ROW_BIT) & 1) << 5); };
+        __syncthreads(); // every wave is done with the stages: the images reuse their memory
+        float* image = lds + wk * (BM * BN);
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+#pragma unroll
+            for(int v = 0; v < ACC; ++v)
+            {
+                const int r = wm0 + impl::tile_index<X_KC, VM, MI>(i, impl::acc_row<MI>(v, h_e));
+                if constexpr(!Y_KC && VN > 1)
+                {
+                    // a lane's VN tiles are adjacent columns: one 64- or 128-bit write, contiguous
+                    // across the lanes
+#pragma unroll
+                    for(int g = 0; g < TN / VN; ++g)
+                    {
+                        float* dst = image + image_index(r, wn0 + g * MI * VN + VN * c_e);
+                        if constexpr(VN == 4)
+                            *reinterpret_cast<f32x4*>(dst)
+                                = f32x4{acc[i][g * 4 + 0][v], acc[i][g * 4 + 1][v], acc[i][g * 4 + 2][v], acc[i][g * 4 + 3][v]};
+                        else
+                            *reinterpret_cast<f32x2*>(dst) = f32x2{acc[i][g * 2 + 0][v], acc[i][g * 2 + 1][v]};
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for(int j = 0; j < TN; ++j)
+                        image[image_index(r, wn0 + impl::tile_index<Y_KC, VN, MI>(j, c_e))] = acc[i][j][v];
+                }
+            }
+        __syncthreads();
+#pragma unroll
+        for(int g = 0; g < NSUM; ++g)
+        {
+            const int p = (g * NT + tid) * 4; // linear position: consecutive threads, consecutive banks
+            f32x4     o = *reinterpret_cast<const f32x4*>(lds + p);
+#pragma unroll
+            for(int w = 1; w < WK; ++w)
+                o += *reinterpret_cast<const f32x4*>(lds + w * (BM * BN) + p);
+            summed[g] = o;
+        }
     }
-    } // WK == 1
+
+    // (Only kernels of at most four waves that each own at most a 64 x 64 share of the tile can sum
+    // in the launch: with a larger share one wave would have too much to add up, and the code
+    // would not fit next to 128 or 256 accumulators without spilling.  The host never passes
+    // counters to the others.)
+    if(!Cfg::SUMS_IN_LAUNCH || !to_partial || args.counters == nullptr)
+    {
+        // the tile is final, or a second kernel sums the partial tiles
+        put_tile(mine);
+    }
+    else if constexpr(Cfg::SUMS_IN_LAUNCH)
+    {
+        // Partial tile, summed in this launch.  Every wave shares its part of the tile, then takes
+        // a ticket from the counter of (tile, wave position); the wave that draws the last ticket
+        // knows that every other part is complete in memory, adds them all up in a fixed order -
+        // K slices in slice order, tail segments in workgroup order - and stores the result.  No
+        // wave ever waits for another.
+        // Ordering.  Writers: the parts are stored with the agent-scope cache policy; the fence makes
+        // the wave wait until those stores are complete (and keeps the compiler from moving them)
+        // before the ticket is drawn.  Reader: the parts are read with the same policy by loads
+        // issued after the ticket has come back, so no cache can hand out a line that is older than
+        // the ticket.
+        share_tile(mine);
+        const int tile_id  = tail ? tail_u0 + seg : wg; // tail: number of the tail tile; else the tile
+        const int expected = tail ? min(((tile_id + 1) * k_tiles - 1) / args.tail_per, args.tail_groups - 1)
+                                        - (tile_id * k_tiles) / args.tail_per + 1
+                                  : args.split_k;
+        unsigned* counter = args.counters
+                            + (static_cast<size_t>(batch) * (tail ? tiles - args.tail_begin : tiles) + tile_id) * (NT / 64)
+                            + wave;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        unsigned ticket = 0;
+        if(lane == 0)
+        {
+            ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if(static_cast<int>(ticket) == expected - 1)
+        {
+            if(lane == 0)
+            {
+                // left at zero for the next launch that uses the counter (stream order separates them)
+                __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if(tail)
+            {
+                const int g_first = (tile_id * k_tiles) / args.tail_per;
+                sum_parts(expected, [&](int n) {
+                    const int g = g_first + n;
+                    return segment_place(g, (g * args.tail_per) / k_tiles == tile_id ? 0 : 1);
+                });
+            }
+            else
+            {
+                sum_parts(args.split_k, slice_place);
+            }
+        }
+    }
     if(seg + 1 < nseg)
     {
         // the next segment refills the LDS stages: every wave must be done reading them

@@ -97,11 +97,12 @@ EDGE_SHAPES = [(1, 1, 1), (33, 65, 17), (255, 257, 129), (300, 260, 100), (64, 6
 @pytest.mark.parametrize("la,lb,lc", ALL_LAYOUTS, ids=LAYOUT_IDS)
 def test_every_kernel_exact_on_integers(la, lb, lc):
     rng = np.random.default_rng(100 + la * 4 + lb * 2 + lc)
-    # (split_k, wave_slots): plain, uniform split-K, and a tail split forced by pretending the GPU
-    # runs only 3 workgroups at once
+    # (split_k, wave_slots, partial_sums): plain, uniform split-K, and a tail split forced by
+    # pretending the GPU runs only 3 workgroups at once - the last two with the partial tiles
+    # summed by a second kernel (1) and by the GEMM launch itself where the kernel can (2)
     for fam in rs.family():
-        for split, slots in ((1, 1), (3, 1), (1, 3)):
-            cfg = dict(fam.as_dict(), split_k=split, group_m=3, wave_slots=slots)
+        for split, slots, sums in ((1, 1, 0), (3, 1, 1), (3, 1, 2), (1, 3, 1), (1, 3, 2)):
+            cfg = dict(fam.as_dict(), split_k=split, group_m=3, wave_slots=slots, partial_sums=sums)
             for (M, N, K) in EDGE_SHAPES:
                 _announce("int_exact", cfg, M, N, K, la, lb, lc)
                 check_exact_int(M, N, K, la, lb, lc, rng, cfg)
@@ -490,6 +491,34 @@ def test_sixteen_byte_loads_that_straddle_the_end_of_a_padded_operand():
             check_strided_batched_exact(rng, M, N, K, la, lb, lc, 1, 1, 0, pads, config=cfg)
 
 
+def test_partial_tiles_summed_in_the_launch_equal_the_second_kernel_bit_for_bit():
+    """The parts of a tile are added in the same order whoever adds them - the wave that draws the
+    last ticket inside the GEMM launch, or the reduction kernel - so uniform inputs must give the
+    same bits, call after call (the counters of a launch are left at zero for the next one, and the
+    workspace is reused with other contents in between)."""
+    import torch
+    fams = {(f.macro_m, f.macro_n, f.k_tile, f.waves_k): f for f in rs.family() if f.stages >= 2 and f.mfma == 32}
+    cases = [((64, 64, 64, 4), (768, 384, 2304), dict(split_k=3, wave_slots=1)),
+             ((64, 32, 64, 4), (300, 777, 4100), dict(split_k=5, wave_slots=1)),
+             ((128, 128, 32, 1), (1000, 1100, 2048), dict(split_k=1, wave_slots=7)),
+             ((64, 64, 32, 1), (1030, 2050, 777), dict(split_k=2, wave_slots=1)),
+             ((128, 64, 32, 2), (382, 1059, 3350), dict(split_k=1, wave_slots=0)),
+             ((64, 64, 128, 4), (1024, 1024, 4096), dict(split_k=2, wave_slots=1))]
+    for key, (M, N, K), launch in cases:
+        dA, dB = _device_uniform(M, K, M + 1), _device_uniform(K, N, N + 2)
+        outs = []
+        for sums in (1, 2, 2, 1, 2):
+            cfg = dict(fams[key].as_dict(), group_m=4, partial_sums=sums, **launch)
+            _announce("partial_sums", cfg, M, N, K)
+            dC = torch.full((M * N,), float("nan"), dtype=torch.float32, device="cuda:0")
+            rs.gemm_with_config(cfg, dC, dA, dB, M, N, K, stream=torch.cuda.current_stream())
+            torch.cuda.synchronize()
+            outs.append(dC)
+        for other in outs[1:]:
+            assert torch.equal(outs[0].view(torch.int32), other.view(torch.int32)), (key, M, N, K)
+        _sampled_check(dA, dB, outs[1], M, N, K, 0, 0, 0)
+
+
 def test_stream_k_tail_matches_plain_run_and_is_deterministic():
     """The stream-K tail (K range of a short last wave of tiles dealt out to all slots) changes
     only the summation order of the affected tiles: results stay within the fp64 tolerance, repeat
@@ -539,7 +568,7 @@ def test_concurrent_calls_from_threads_on_separate_streams():
     small = [f for f in rs.family() if f.macro_m == 64 and f.macro_n == 64][0].as_dict()
     for idx, (shape, cfg) in enumerate([((512, 384, 640), dict(base)),
                                          ((300, 260, 1000), dict(base, split_k=4)),
-                                         ((260, 300, 520), dict(small, wave_slots=7)),
+                                         ((260, 300, 520), dict(small, wave_slots=7, partial_sums=2)),
                                          ((129, 1000, 77), dict(small))]):
         M, N, K = shape
         A = rng.integers(-4, 5, size=(M, K)).astype(np.float32)

@@ -87,7 +87,7 @@ def _py_plan(table, M, N, K, a, b, c):
     """Restatement of the planning rule around the library's own cost model: table entries are
     returned as they are; otherwise the nearest entry's config, unless one of the four nearest
     entries of the same layouts and kind (split_k fitted first) or one of the larger direct-to-LDS
-    tile shapes (or smaller ones with waves along K) at split_k 1, 2, 4 or 8 is predicted at least
+    tile shapes (or smaller ones with waves along K) at split_k 1, 2, 3, 4, 6 or 8 is predicted at least
     4 % faster."""
     nearest = _py_select(table, M, N, K, a, b, c).as_dict()
     if any(key == (M, N, K, a, b, c) for key, _ in table):
@@ -108,7 +108,7 @@ def _py_plan(table, M, N, K, a, b, c):
         if fam.stages < 2 or fam.mfma != 32 or ((fam.macro_m < 64 or fam.macro_n < 64) and fam.waves_k <= 1):
             continue
         k_tiles = -(-K // fam.k_tile)
-        for split in (1, 2, 4, 8):
+        for split in (1, 2, 3, 4, 6, 8):
             if split > 1 and k_tiles < 2 * split:
                 break
             candidates.append(dict(fam.as_dict(), split_k=split, group_m=4, wave_slots=0))
@@ -344,8 +344,8 @@ def test_space_constraints():
     assert space.shape_ok((64, 64, 64, 1, 1, 32, 2, 4))
     assert not space.shape_ok((64, 64, 64, 1, 1, 32, 0, 4))
     assert not space.shape_ok((64, 64, 32, 1, 1, 32, 2, 4))  # one k-block per wave
-    assert not space.shape_ok((256, 256, 32, 2, 4, 32, 2, 2))  # 2 x 256 x 264 floats > 160 KB
-    assert space.lds_bytes(64, 64, 64, 1, 0, 2, 4) == 4 * 64 * 72 * 4
+    assert not space.shape_ok((256, 256, 32, 2, 4, 32, 2, 2))  # 2 x 256 x 256 floats > 160 KB
+    assert space.lds_bytes(64, 64, 32, 1, 0, 2, 4) == 4 * 64 * 64 * 4  # the images, more than the stages
 
 
 def test_generator_outputs(tmp_path):
@@ -414,9 +414,9 @@ def _fake_runner(best_shape, best_group):
                 for sp in splits:
                     for g in groups:
                         ms = 1.0 if (s == best_shape and sp == 1) else 2.0
-                        lines.append("cfg " + " ".join(map(str, s[:7] + (sp, g, 0, s[7])))
+                        lines.append("cfg " + " ".join(map(str, s[:7] + (sp, g, 0, s[7], 0)))
                                      + f" avg_ms {ms:.4f} min_ms {ms:.4f} tflops 1.00 ok 1")
-            lines.append("cfg 32 32 32 1 1 32 0 1 4 0 1 avg_ms 0.0100 min_ms 0.0100 tflops 9.00 ok 0")
+            lines.append("cfg 32 32 32 1 1 32 0 1 4 0 1 0 avg_ms 0.0100 min_ms 0.0100 tflops 9.00 ok 0")
             return _FakeProc("\n".join(lines))
         cfg = dict(zip(space.CONFIG_KEYS, map(int, cmd[4:4 + len(space.CONFIG_KEYS)])))
         shape = tuple(cfg[k] for k in space.SHAPE_KEYS)

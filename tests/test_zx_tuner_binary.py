@@ -40,7 +40,7 @@ def test_single_config_mode_times_and_verifies_one_trial():
     avg_ms, min_ms, tflops = map(float, m.groups())
     assert 0.0 < min_ms <= avg_ms * 1.5 and avg_ms < 5.0 and tflops > 0.5
     # a tile shape that is not compiled is refused, as the reference's launcher refuses a null slot
-    bad = [TUNER, str(M), str(N), str(K), "96", "96", "32", "2", "2", "32", "2", "1", "4", "0", "1", "0", "0", "0"]
+    bad = [TUNER, str(M), str(N), str(K), "96", "96", "32", "2", "2", "32", "2", "1", "4", "0", "1", "0", "0", "0", "0"]
     refused = subprocess.run(bad, capture_output=True, text=True, timeout=120)
     assert refused.returncode == 3 and "No kernel available" in refused.stderr
 

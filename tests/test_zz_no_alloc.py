@@ -32,9 +32,11 @@ def _needs_scratch(M, N, K):
 def test_no_alloc_entry_equals_the_allocating_entry_on_calls_in_a_row():
     import torch
     stream = torch.cuda.current_stream()
-    # deep K (split-K, 32 MiB of partials), a stream-K tail, then two smaller split-K problems
-    shapes = [(1024, 1024, 16384), (2560, 2560, 2560), (128, 4096, 4096), (300, 260, 4096)]
+    # deep K (split-K, 32 MiB of partials), a stream-K tail, then smaller split-K problems (summed
+    # by a second kernel, by the launch itself, and ragged)
+    shapes = [(1024, 1024, 16384), (2560, 2560, 2560), (512, 512, 8192), (300, 260, 4096), (32, 4096, 4096)]
     assert _needs_scratch(*shapes[0]) > _needs_scratch(*shapes[2]) > 0
+    assert _needs_scratch(*shapes[3]) > 0 and _needs_scratch(*shapes[4]) > 0
     for (M, N, K) in shapes:
         print("CASE no_alloc", M, N, K, rs.find_config(M, N, K), flush=True)
         g = torch.Generator(device="cuda:0")
@@ -66,7 +68,7 @@ def test_no_alloc_entry_in_column_major_layouts_and_on_a_side_stream():
     rng = np.random.default_rng(10)
     side = torch.cuda.Stream()
     for (la, lb, lc) in [(1, 1, 1), (0, 1, 0), (1, 0, 1)]:
-        M, N, K = 128, 4096, 2048
+        M, N, K = 32, 4096, 4096
         print("CASE no_alloc layouts", M, N, K, la, lb, lc, flush=True)
         A, B, C = int_matrices(rng, M, N, K)
         a = A.reshape(-1) if la == 0 else A.T.reshape(-1)
