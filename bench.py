@@ -14,15 +14,20 @@ back and the region is closed by one device synchronisation.
 
 Also in the line:
   roofline      MFMA-bound: achieved = 2MNK / mean launch duration, peak = 157.3 TFLOP/s (dense FP32
-                matrix peak of MI355X); traffic = measured HBM bytes per launch if a counter summary
-                is available under profiles/ (written by --counters), else null
-  layouts       avg / min TFLOP/s of the four A/B storage combinations (NN/NT/TN/TT) with C row- and
-                column-major, uniform[-1, 1) A and B, at 4096^3 and 8192^3
+                matrix peak of MI355X); traffic = HBM bytes per launch measured by --counters in this
+                run, else read from the summary an earlier --counters run left under profiles/
+                (traffic_source says which), else null
+  layouts       the reference bench's default cubes, 1024^3 to 8192^3, in the four A/B storage
+                combinations (NN/NT/TN/TT) with C row- and column-major, uniform[-1, 1) A and B.
+                Per row: avg / min-time TFLOP/s of the per-launch event pairs, the sustained rate
+                (first start event to last stop event) and the back-to-back rate (one event pair
+                around the same number of launches: no event packets between the kernels)
   shapes_row_major  the rectangular, unaligned and 16384^3 row-major configurations, with the
-                vendor library on the same operands beside them
+                vendor library on the same operands, by the same protocol, beside them
   context       hipBLASLt / rocBLAS (through torch.matmul, fp32, TF32 off) on the same GPU
-  cpu_baseline  the reference's CPU GEMM (the oracle's restatement of sgemm_cpu, single thread, as
-                the reference runs it) on a bounded 1024^3 sample, timed on this host; plus, where
+  cpu_baseline  the reference's CPU GEMM (the oracle's restatement of sgemm_cpu): one thread at
+                1024^3 as the reference runs it, all usable threads at 1024^3 and on a bounded
+                sample of 4096^3 (labelled extrapolated when cut), timed on this host; plus, where
                 it has been built, the reference's own GPU kernel on this GPU for context
 --counters additionally runs the timed loop under rocprofv3 --pmc (MFMA busy, LDS bank conflicts,
 HBM bytes) and writes profiles/sgemm_mfma_4096_rrr_counters.txt.
@@ -53,13 +58,16 @@ def tflops(m, n, k, ms):
     return 2.0 * m * n * k / (ms * 1e-3) * 1e-12
 
 
-WARMUP_MIN_MS = 40.0  # sustained launches before any timed region (the clocks need tens of ms)
+WARMUP_MIN_MS = 40.0   # sustained launches before any timed region (the clocks need tens of ms)
+WARMUP_MAX_MS = 600.0  # ... and at most this long while the launch time is still falling
 
 
-def timed_launches(fn, steps, warmup, min_warm_ms=WARMUP_MIN_MS):
+def timed_launches(fn, steps, warmup, min_warm_ms=WARMUP_MIN_MS, max_warm_ms=WARMUP_MAX_MS):
     """The one timing protocol of this file.  Warm-up: at least `warmup` launches AND at least
-    `min_warm_ms` of sustained launches (after an idle gap the GPU needs tens of milliseconds of
-    work to reach its full clock, whatever the launch count).  Then `steps` launches queued back to
+    `min_warm_ms` of sustained launches, continued in batches of about 10 ms until two batches in
+    a row agree within 1 % (after an idle gap the GPU needs tens of milliseconds of work to reach
+    its full clock, more for some kernels: 1024 x 1024 x 16384 launches fell from 302 to 245 us
+    over the 100 launches that followed a 40 ms warm-up).  Then `steps` launches queued back to
     back, each bracketed by an event pair on the launch stream, closed by ONE synchronisation.
     Returns the per-launch durations (ms), the wall time (ms) of the timed region, and the device
     time (ms) from the first launch's start event to the last one's stop event - the sustained
@@ -67,9 +75,9 @@ def timed_launches(fn, steps, warmup, min_warm_ms=WARMUP_MIN_MS):
     import torch
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]  # before the warm-up:
     stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]   # no idle gap after it
-    warmed_ms, launched, batch = 0.0, 0, 5
+    warmed_ms, launched, batch, previous = 0.0, 0, 5, None
     w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    while launched < warmup or warmed_ms < min_warm_ms:
+    while True:
         w0.record()
         for _ in range(batch):
             fn()
@@ -78,9 +86,13 @@ def timed_launches(fn, steps, warmup, min_warm_ms=WARMUP_MIN_MS):
         took = max(w0.elapsed_time(w1), 1e-3)
         warmed_ms += took
         launched += batch
-        # next batch: what is left of the warm-up time at the rate just seen
-        left = max(min_warm_ms - warmed_ms, 0.0) * batch / took
-        batch = int(max(warmup - launched, min(left, 5000), 1))
+        per_launch = took / batch
+        settled = previous is not None and abs(per_launch - previous) <= 0.01 * previous
+        previous = per_launch
+        if launched >= warmup and warmed_ms >= min_warm_ms and (settled or warmed_ms >= max_warm_ms):
+            break
+        # next batch: about 10 ms at the rate just seen (at least what `warmup` still asks for)
+        batch = int(max(warmup - launched, min(10.0 / per_launch, 5000), 2))
     t0 = time.perf_counter()
     for i in range(steps):
         starts[i].record()
@@ -91,13 +103,36 @@ def timed_launches(fn, steps, warmup, min_warm_ms=WARMUP_MIN_MS):
     return [s.elapsed_time(e) for s, e in zip(starts, stops)], wall_ms, starts[0].elapsed_time(stops[-1])
 
 
-def summary(m, n, k, ms, span_ms):
+def summary(m, n, k, ms, span_ms, burst_ms=None):
     avg = sum(ms) / len(ms)
-    return {"avg_tflops": round(tflops(m, n, k, avg), 2),
-            "min_time_tflops": round(tflops(m, n, k, min(ms)), 2),
-            "pct_peak_avg": round(100 * tflops(m, n, k, avg) / PEAK_TFLOPS, 1),
-            "avg_ms": round(avg, 5),
-            "sustained_tflops": round(tflops(m, n, k, span_ms / len(ms)), 2)}
+    out = {"avg_tflops": round(tflops(m, n, k, avg), 2),
+           "min_time_tflops": round(tflops(m, n, k, min(ms)), 2),
+           "pct_peak_avg": round(100 * tflops(m, n, k, avg) / PEAK_TFLOPS, 1),
+           "avg_ms": round(avg, 5),
+           "sustained_tflops": round(tflops(m, n, k, span_ms / len(ms)), 2)}
+    if burst_ms is not None:
+        out["back_to_back_tflops"] = round(tflops(m, n, k, burst_ms), 2)
+        out["back_to_back_ms"] = round(burst_ms, 5)
+    return out
+
+
+def burst_ms(fn, steps):
+    """Mean duration of `steps` launches queued back to back between ONE event pair (right after
+    a timed region, so the GPU is warm): no event packets between the kernels, which cost a few
+    microseconds each - what a caller that just issues products sees."""
+    import torch
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def measure(fn, m, n, k, steps, warmup):
+    ms, _, span = timed_launches(fn, steps, warmup)
+    return summary(m, n, k, ms, span, burst_ms(fn, steps))
 
 
 def uniform_device(count, seed):
@@ -123,9 +158,8 @@ def bench_layouts(rs, sizes, steps, warmup):
                 for lb in (0, 1):
                     def fn():
                         rs.gemm(dC, dA, dB, size, size, size, lc, la, lb, stream=stream)
-                    ms, _, span = timed_launches(fn, n_steps, warmup)
                     key = f"{size}^3 A={names[la]} B={names[lb]} C={names[lc]}"
-                    out[key] = summary(size, size, size, ms, span)
+                    out[key] = measure(fn, size, size, size, n_steps, warmup)
         del dA, dB, dC
     return out
 
@@ -146,12 +180,12 @@ def bench_shapes(rs, steps, warmup):
         dC = torch.empty(m * n, dtype=torch.float32, device="cuda:0")
         flop_ms = 2.0 * m * n * k / 140e9  # rough duration, to keep every shape to a fraction of a second
         n_steps = max(5, min(steps, int(200 / max(flop_ms, 0.01))))
-        ms, _, span = timed_launches(lambda: rs.gemm(dC, dA, dB, m, n, k, stream=stream), n_steps, warmup)
+        row = measure(lambda: rs.gemm(dC, dA, dB, m, n, k, stream=stream), m, n, k, n_steps, warmup)
         a2, b2 = dA.view(m, k), dB.view(k, n)
-        vms, _, vspan = timed_launches(lambda: torch.matmul(a2, b2), n_steps, warmup)
-        row = summary(m, n, k, ms, span)
-        row["vendor_avg_tflops"] = round(tflops(m, n, k, sum(vms) / len(vms)), 2)
-        row["vendor_sustained_tflops"] = round(tflops(m, n, k, vspan / len(vms)), 2)
+        vendor = measure(lambda: torch.matmul(a2, b2), m, n, k, n_steps, warmup)
+        row["vendor_avg_tflops"] = vendor["avg_tflops"]
+        row["vendor_sustained_tflops"] = vendor["sustained_tflops"]
+        row["vendor_back_to_back_tflops"] = vendor["back_to_back_tflops"]
         row["kernel_config"] = rs.find_config(m, n, k).as_dict()
         out[f"{m}x{n}x{k}"] = row
         del dA, dB, dC, a2, b2
@@ -167,8 +201,8 @@ def bench_context(sizes, steps, warmup):
         a = uniform_device(size * size, 3).view(size, size)
         b = uniform_device(size * size, 4).view(size, size)
         n_steps = steps if size <= 4096 else max(10, steps // 5)
-        ms, _, span = timed_launches(lambda: torch.matmul(a, b), n_steps, warmup)
-        out[f"torch.matmul fp32 {size}^3 (hipBLASLt/rocBLAS)"] = summary(size, size, size, ms, span)
+        out[f"torch.matmul fp32 {size}^3 (hipBLASLt/rocBLAS)"] = measure(lambda: torch.matmul(a, b), size, size, size,
+                                                                          n_steps, warmup)
     return out
 
 

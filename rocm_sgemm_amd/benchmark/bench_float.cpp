@@ -222,9 +222,12 @@ struct timing
 };
 
 // Warm-up is by count AND by time: after an idle gap the GPU takes tens of milliseconds of
-// sustained work to reach its full clock, so at least `warm_ms` of back-to-back launches precede
-// the timed ones whatever `warmup` says (0 under rocprofv3 --pmc, where every launch is costly).
+// sustained work to reach its full clock (more for some kernels), so at least `min_warm_ms` of
+// back-to-back launches precede the timed ones whatever `warmup` says, continued in batches of
+// about 10 ms until two batches in a row agree within 1 % or `max_warm_ms` have passed (0 under
+// rocprofv3 --pmc, where every launch is costly).
 double min_warm_ms = 40.0;
+double max_warm_ms = 600.0;
 
 template<class Launch>
 timing time_launches(Launch&& launch, hipStream_t stream, int warmup, int iters, double flops)
@@ -235,8 +238,8 @@ timing time_launches(Launch&& launch, hipStream_t stream, int warmup, int iters,
     for(int i = 0; i < warmup; ++i)
         launch();
     HIP_CHECK(hipStreamSynchronize(stream));
-    double warmed_ms = 0.0;
-    for(int batch = 4; warmed_ms < min_warm_ms;)
+    double warmed_ms = 0.0, previous = -1.0;
+    for(int batch = 4; min_warm_ms > 0.0;)
     {
         HIP_CHECK(hipEventRecord(e0, stream));
         for(int i = 0; i < batch; ++i)
@@ -246,8 +249,12 @@ timing time_launches(Launch&& launch, hipStream_t stream, int warmup, int iters,
         float ms = 0;
         HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
         warmed_ms += ms;
-        const double left = (min_warm_ms - warmed_ms) * batch / (ms > 1e-3f ? ms : 1e-3f);
-        batch             = left < 1.0 ? 1 : (left > 4096.0 ? 4096 : static_cast<int>(left));
+        const double per_launch = (ms > 1e-3f ? ms : 1e-3f) / batch;
+        const bool   settled    = previous > 0.0 && std::fabs(per_launch - previous) <= 0.01 * previous;
+        previous                = per_launch;
+        if(warmed_ms >= min_warm_ms && (settled || warmed_ms >= max_warm_ms)) break;
+        const double next = 10.0 / per_launch;
+        batch             = next < 2.0 ? 2 : (next > 4096.0 ? 4096 : static_cast<int>(next));
     }
     timing t;
     t.min_ms            = std::numeric_limits<double>::max();
@@ -652,8 +659,8 @@ int run(const options& opt)
     HIP_CHECK(hipGetDeviceProperties(&prop, 0));
     std::printf("device: %s %s, %d CUs, %d MHz; peak used for pct_peak: %.1f TFLOP/s (dense FP32 matrix)\n",
                 prop.name, prop.gcnArchName, prop.multiProcessorCount, prop.clockRate / 1000, peak_tflops);
-    std::printf("protocol: %d warm-up launches (and at least %.0f ms of them) + %d timed launches per row, one event "
-                "pair per launch, each waited for; inputs: %s\n",
+    std::printf("protocol: %d warm-up launches (and at least %.0f ms of them, until the launch time has settled) + %d "
+                "timed launches per row, one event pair per launch, each waited for; inputs: %s\n",
                 opt.warmup, min_warm_ms, opt.iters,
                 opt.identity_b ? "A uniform[-1,1), B = identity"
                                : (opt.uniform ? "uniform[-1,1)" : "cyclic {1.025,1.05,1.075,1.1,1.0}"));
@@ -909,10 +916,10 @@ int run_host_cost()
         std::printf("host_cost call  %-58s %8.3f us per call   (first shape: split_k %d)\n", what, total / rounds,
                     cfg.split_k);
     };
-    call_cost("plain product, one launch (256^3)", {{256, 256, 256}});
-    call_cost("plain product, one launch (1024^3)", {{1024, 1024, 1024}});
-    call_cost("split-K product, two launches (1024 x 1024 x 16384)", {{1024, 1024, 16384}});
-    call_cost("stream-K tail, two launches (2560^3)", {{2560, 2560, 2560}});
+    call_cost("plain product (256^3)", {{256, 256, 256}});
+    call_cost("plain product (1024^3)", {{1024, 1024, 1024}});
+    call_cost("split-K product (1024 x 1024 x 16384)", {{1024, 1024, 16384}});
+    call_cost("stream-K tail (2560^3)", {{2560, 2560, 2560}});
     call_cost("two planned shapes in turn", {{1536, 1200, 900}, {777, 2222, 1111}});
     call_cost("twenty planned shapes in turn", many);
     HIP_CHECK(hipFree(dA));

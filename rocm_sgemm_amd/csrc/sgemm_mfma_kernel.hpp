@@ -179,6 +179,14 @@ struct tile_config
     static constexpr int EX_FLOATS  = WK > 1 ? WK * BM * BN : 0;
     static constexpr int LDS_FLOATS = STAGES * STAGE > EX_FLOATS ? STAGES * STAGE : EX_FLOATS;
     static constexpr int LDS_BYTES = LDS_FLOATS * 4;
+    // Waves per SIMD the register allocator is held to.  Left to itself it sizes a kernel for one
+    // workgroup per CU; a K-split kernel whose LDS lets two workgroups share a CU (128 x 64 and
+    // 64 x 128 with WK = 2) then takes 264 - 270 registers for the summing code of the epilogue,
+    // just over the 256 that two waves per SIMD leave each, and loses 5 % (2048^3: 131.6 against
+    // 137.8 TFLOP/s).  Only those kernels are bounded; the others fit as they are.
+    static constexpr int WG_PER_CU_BY_LDS = 160 * 1024 / LDS_BYTES;
+    static constexpr int MIN_WAVES_PER_SIMD
+        = WK > 1 && WG_PER_CU_BY_LDS >= 2 && BM * BN / (WM * WN) >= 64 * 64 ? 2 * ((NT / 64 + 3) / 4) : 1;
 
     // Swizzle of a depth-contiguous direct-to-LDS image: rows of BK floats, CPR 16-byte chunks
     // each, RPL rows per 64-bank line.
@@ -552,7 +560,7 @@ __device__ __forceinline__ constexpr int acc_row(int v, int h)
 } // namespace impl
 
 template<class Cfg>
-__global__ __launch_bounds__(Cfg::NT) void sgemm_mfma_kernel(const gemm_args args)
+__global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_kernel(const gemm_args args)
 {
     constexpr int  BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
     constexpr int  TM = Cfg::TM, TN = Cfg::TN, NT = Cfg::NT, NKB = Cfg::NKBW, WK = Cfg::WK;
