@@ -576,3 +576,37 @@ def test_sampled_check_fails_on_nan_and_unwritten_outputs(tmp_path):
                     str(src), "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
     assert out == ["1", "0", "0", "0"], out
+
+
+def test_no_kernel_spills_and_registers_leave_the_occupancy_that_lds_allows(tmp_path):
+    """Reads the register, LDS and scratch sizes of every compiled GEMM kernel from the library's
+    code-object metadata.  A kernel that spills, or whose register count halves the number of
+    workgroups its LDS footprint lets a CU hold, still computes the right product, only slower;
+    no parity test sees that."""
+    bundler, readelf = "/opt/rocm/llvm/bin/clang-offload-bundler", "/opt/rocm/llvm/bin/llvm-readelf"
+    if not (os.path.exists(bundler) and os.path.exists(readelf)):
+        pytest.skip("needs the ROCm LLVM tools")
+    fat = tmp_path / "fat.bin"
+    subprocess.run(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", rs.lib_path(), str(fat)], check=True)
+    data = fat.read_bytes()
+    starts = [m.start() for m in re.finditer(b"__CLANG_OFFLOAD_BUNDLE__", data)] + [len(data)]
+    kernels = []
+    for a, b in zip(starts, starts[1:]):
+        (tmp_path / "bundle").write_bytes(data[a:b])
+        subprocess.run([bundler, "--unbundle", "--type=o", f"--input={tmp_path / 'bundle'}",
+                        "--targets=hipv4-amdgcn-amd-amdhsa--gfx950", f"--output={tmp_path / 'co'}"], check=True)
+        notes = subprocess.run([readelf, "--notes", str(tmp_path / "co")], capture_output=True, text=True).stdout
+        for block in notes.split("- .agpr_count:")[1:]:
+            field = lambda key: re.search(rf"\.{key}:\s*(\S+)", block).group(1)  # noqa: E731
+            kernels.append((field("name"), int(field("vgpr_count")), int(field("group_segment_fixed_size")),
+                            int(field("private_segment_fixed_size")), int(field("max_flat_workgroup_size"))))
+    gemm = [k for k in kernels if "sgemm_mfma_kernel" in k[0]]
+    assert len(gemm) >= 4 * sum(3 if s[6] else 2 for s in space.family())
+    for name, registers, lds, scratch, threads in gemm:
+        assert scratch == 0, (name, scratch)
+        waves = threads // 64
+        groups_by_lds = min(160 * 1024 // lds, 8)
+        waves_per_simd = 512 // ((registers + 7) // 8 * 8)  # VGPRs and AGPRs share 512 per lane
+        groups_by_registers = waves_per_simd * 4 // waves if waves <= 4 else waves_per_simd // (waves // 4)
+        # register-staged kernels keep their staging registers; two workgroups per CU is their design point
+        assert groups_by_registers >= min(groups_by_lds, 2), (name, registers, lds)
