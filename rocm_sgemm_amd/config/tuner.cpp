@@ -95,6 +95,7 @@ bool verify(const problem& p)
 }
 
 constexpr double warmup_min_ms = 40.0;
+constexpr double warmup_max_ms = 600.0;
 
 struct timing
 {
@@ -109,33 +110,58 @@ timing run_trial(problem& p, const rocm_sgemm_config& cfg, int iters, int warmup
     CHECK_HIP(hipEventCreate(&e0));
     CHECK_HIP(hipEventCreate(&e1));
     CHECK_HIP(hipMemsetAsync(p.dC, 0xFF, p.M * p.N * sizeof(float), p.stream));
-    // Warm-up is by count AND by time: after an idle gap the GPU takes tens of milliseconds of
-    // sustained work to reach its full clock, and a trial timed before that is pessimistic.
     const auto launch = [&]() {
         return rocm_sgemm_f32_with_config(&cfg, p.lc, p.la, p.lb, p.dC, p.dA, p.dB, p.M, p.N, p.K,
                                           p.stream);
     };
-    double warmed_ms = 0.0;
-    for(int i = 0; i < warmup || warmed_ms < warmup_min_ms; ++i)
+    // Warm-up is by count AND by time: after an idle gap (the start of the process, the check of
+    // the previous trial) the GPU takes tens of milliseconds of sustained work to reach its full
+    // clock, some kernels several hundred, and a trial timed before that is pessimistic by an
+    // amount that differs from config to config (1024 x 1024 x 16384: up to 10 %, enough to rank
+    // two configs the wrong way round).  So launches are queued back to back in batches of about
+    // 10 ms until at least warmup_min_ms have passed and two batches in a row agree within 1 %
+    // (or warmup_max_ms have passed).
+    if(launch() != ROCM_SGEMM_STATUS_OK)
+    {
+        std::fprintf(stderr, "trial rejected: %s\n", rocm_sgemm_last_error());
+        CHECK_HIP(hipEventDestroy(e0));
+        CHECK_HIP(hipEventDestroy(e1));
+        return r;
+    }
+    for(int i = 1; i < warmup; ++i)
+    {
+        launch();
+    }
+    CHECK_HIP(hipStreamSynchronize(p.stream));
+    double warmed_ms = 0.0, previous = -1.0;
+    for(int batch = 4;;)
     {
         CHECK_HIP(hipEventRecord(e0, p.stream));
-        if(launch() != ROCM_SGEMM_STATUS_OK)
+        for(int i = 0; i < batch; ++i)
         {
-            std::fprintf(stderr, "trial rejected: %s\n", rocm_sgemm_last_error());
-            CHECK_HIP(hipEventDestroy(e0));
-            CHECK_HIP(hipEventDestroy(e1));
-            return r;
+            launch();
         }
         CHECK_HIP(hipEventRecord(e1, p.stream));
         CHECK_HIP(hipEventSynchronize(e1));
         float ms = 0.0f;
         CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
         warmed_ms += ms;
+        const double per_launch = (ms > 1e-3f ? ms : 1e-3f) / batch;
+        const bool   settled    = previous > 0.0 && std::fabs(per_launch - previous) <= 0.01 * previous;
+        previous                = per_launch;
+        if(warmed_ms >= warmup_min_ms && (settled || warmed_ms >= warmup_max_ms))
+        {
+            break;
+        }
+        const double next = 10.0 / per_launch;
+        batch             = next < 2.0 ? 2 : (next > 4096.0 ? 4096 : static_cast<int>(next));
     }
     // Timed region: `iters` launches queued back to back, closed by one synchronisation - the
     // sustained rate a caller issuing GEMM after GEMM sees.  (With a host wait after every launch
     // the GPU idles between kernels, boosts its clock and favours other configs.)  The minimum is
     // taken over a few single launches timed the same way afterwards.
+    // (at least 5 ms of them: thirty launches of a 20 us kernel are over before the timer's noise is)
+    iters = std::max(iters, std::min(4096, static_cast<int>(5.0 / previous)));
     CHECK_HIP(hipEventRecord(e0, p.stream));
     for(int i = 0; i < iters; ++i)
     {
