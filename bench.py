@@ -24,7 +24,8 @@ Also in the line:
                 around the same number of launches: no event packets between the kernels)
   shapes_row_major  the rectangular, unaligned and 16384^3 row-major configurations, with the
                 vendor library on the same operands, by the same protocol, beside them
-  context       hipBLASLt / rocBLAS (through torch.matmul, fp32, TF32 off) on the same GPU
+  context       hipBLASLt / rocBLAS (through torch.matmul, fp32, TF32 off) on the same GPU, and
+                the rate of a kernel that issues MFMAs only (the ceiling of this GPU sample)
   cpu_baseline  the reference's CPU GEMM (the oracle's restatement of sgemm_cpu): one thread at
                 1024^3 as the reference runs it, all usable threads at 1024^3 and on a bounded
                 sample of 4096^3 (labelled extrapolated when cut), timed on this host; plus, where
@@ -204,6 +205,24 @@ def bench_context(sizes, steps, warmup):
         out[f"torch.matmul fp32 {size}^3 (hipBLASLt/rocBLAS)"] = measure(lambda: torch.matmul(a, b), size, size, size,
                                                                           n_steps, warmup)
     return out
+
+
+def mfma_only_kernel():
+    """What the matrix pipes reach with nothing else to do (`bench_float --mfma_ceiling`: a kernel
+    of MFMAs only, one workgroup per CU) and the shader clock of every XCD meanwhile - the ceiling
+    every SGEMM kernel on this GPU sample works under.  None where the bench program is not built."""
+    import re
+    import subprocess
+    exe = os.path.join(REPO, "rocm_sgemm_amd", "benchmark", "bench_float")
+    if not os.path.exists(exe):
+        return None
+    out = subprocess.run([exe, "--mfma_ceiling"], capture_output=True, text=True, timeout=120)
+    whole = re.search(r"= ([\d.]+) TFLOP/s = ([\d.]+) % of", out.stdout)
+    if out.returncode != 0 or whole is None:
+        return None
+    clocks = [int(v) for v in re.findall(r"shader clock (\d+) MHz", out.stdout)]
+    return {"tflops": float(whole.group(1)), "pct_peak": float(whole.group(2)), "xcd_shader_clock_mhz": clocks,
+            "note": "256 workgroups of 4 waves issuing v_mfma_f32_32x32x2_f32 only; the launch ends with the slowest XCD"}
 
 
 def cpu_baseline(max_seconds=12.0):
@@ -504,6 +523,9 @@ def main():
         line["shapes_row_major"] = bench_shapes(rs, args.steps, args.warmup)
     if not args.no_context:
         line["context"] = bench_context((4096, 8192), args.steps, args.warmup)
+        ceiling = mfma_only_kernel()
+        if ceiling is not None:
+            line["context"]["kernel of MFMAs only (bench_float --mfma_ceiling)"] = ceiling
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

@@ -34,6 +34,8 @@
 //   --host_cost         what a call costs on the host (no counterpart in the reference, whose call
 //                       is one table lookup and one launch): microseconds per
 //                       rocm_sgemm_find_config, and per enqueued call while the GPU has queue space
+//   --mfma_ceiling      what the matrix pipes reach with nothing else to do: a kernel of MFMAs only,
+//                       one workgroup per CU, with the shader clock of every XCD during the run
 //   --pmc               short run for use under rocprofv3 --pmc: 2 warm-up + 5 timed launches and
 //                       one plain 64 MiB copy kernel, whose known traffic calibrates the
 //                       FETCH_SIZE / WRITE_SIZE counters
@@ -104,6 +106,7 @@ struct options
     bool             vendor      = false;
     bool             pmc         = false; // child mode under rocprofv3
     bool             counters    = false; // parent mode: collect counters row by row
+    bool             mfma_ceiling = false; // time the matrix pipes alone instead of the timing table
     bool             host_cost   = false; // host-side cost of a call instead of the timing table
     std::vector<int> layouts; // bit 2 = A col, bit 1 = B col, bit 0 = C col; empty = all eight
 };
@@ -186,6 +189,7 @@ void print_usage(const char* program)
               << "  --pmc              short run (2 warm-up + 5 timed + a copy probe) for use under rocprofv3 --pmc\n"
               << "  --host_cost        host microseconds per call: planning alone, and enqueueing plain / split-K /\n"
               << "                     stream-K-tail products, one shape repeated and several shapes in turn\n"
+              << "  --mfma_ceiling     TFLOP/s of a kernel that issues MFMAs only, and the shader clock of every XCD meanwhile\n"
               << "  --help             Show this help message\n"
               << "\nExamples:\n"
               << "  " << program << " --shapes 512:1024:2048\n"
@@ -365,6 +369,112 @@ void run_copy_probe()
     HIP_CHECK(hipDeviceSynchronize());
     HIP_CHECK(hipFree(a));
     HIP_CHECK(hipFree(b));
+}
+
+// ---- the matrix pipes alone ---------------------------------------------------------------------
+// One workgroup of four waves per CU (the LDS request keeps a second one out), every wave issuing
+// nothing but v_mfma_f32_32x32x2_f32 on four independent accumulator tiles: no loads, no LDS, no
+// barriers.  What this reaches is the ceiling any SGEMM kernel on this GPU sample works under; the
+// published 157.3 TFLOP/s is 256 CUs x 256 flop per cycle x 2.4 GHz, and the XCDs do not all hold
+// 2.4 GHz while their matrix pipes are full.  Each wave records wall-clock (100 MHz) and shader
+// clock stamps around its loop, which gives the shader clock of every XCD during the run.
+constexpr int burn_lds_floats = 33 * 1024; // 132 KB of the CU's 160 KB
+__global__ __launch_bounds__(256) void bench_mfma_burn(unsigned long long* __restrict__ stamps, float* __restrict__ sink,
+                                                       int iters)
+{
+    typedef float f32x16 __attribute__((ext_vector_type(16)));
+    __shared__ float pad[burn_lds_floats];
+    pad[threadIdx.x] = static_cast<float>(threadIdx.x);
+    __syncthreads();
+    const float a = pad[(threadIdx.x * 7) % 256] * 1e-4f + 1.0f;
+    const float b = pad[(threadIdx.x * 13) % 256] * 1e-4f - 1.0f;
+    f32x16      acc[4];
+    for(int j = 0; j < 4; ++j)
+        for(int v = 0; v < 16; ++v)
+            acc[j][v] = 0.0f;
+#if defined(__HIP_DEVICE_COMPILE__)
+    const unsigned long long t0 = wall_clock64(), c0 = clock64();
+    for(int i = 0; i < iters; ++i)
+    {
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[j], 0, 0, 0);
+    }
+    const unsigned long long t1 = wall_clock64(), c1 = clock64();
+    float                    s  = 0.0f;
+    for(int j = 0; j < 4; ++j)
+        for(int v = 0; v < 16; ++v)
+            s += acc[j][v];
+    if(s == 0.123456f) sink[0] = s; // keeps the accumulators alive
+    if(threadIdx.x % 64 == 0)
+    {
+        unsigned long long* o = stamps + (static_cast<size_t>(blockIdx.x) * 4 + threadIdx.x / 64) * 4;
+        o[0]                  = t0;
+        o[1]                  = t1;
+        o[2]                  = c1 - c0;
+        o[3]                  = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 7; // XCC_ID
+    }
+#endif
+}
+
+int run_mfma_ceiling()
+{
+    hipDeviceProp_t prop;
+    HIP_CHECK(hipGetDeviceProperties(&prop, 0));
+    const int           cus = prop.multiProcessorCount, waves = cus * 4;
+    unsigned long long* stamps;
+    float*              sink;
+    HIP_CHECK(hipMalloc(&stamps, sizeof(unsigned long long) * waves * 4));
+    HIP_CHECK(hipMalloc(&sink, sizeof(float)));
+    const int    iters = 40000; // 160 000 MFMAs per wave: about 4.3 ms
+    const double flop  = static_cast<double>(waves) * iters * 4.0 * (2.0 * 32 * 32 * 2);
+    hipEvent_t   e0, e1;
+    HIP_CHECK(hipEventCreate(&e0));
+    HIP_CHECK(hipEventCreate(&e1));
+    for(int i = 0; i < 30; ++i) // warm-up: well over 100 ms of sustained work
+        hipLaunchKernelGGL(bench_mfma_burn, dim3(cus), dim3(256), 0, nullptr, stamps, sink, iters);
+    HIP_CHECK(hipEventRecord(e0, nullptr));
+    const int launches = 10;
+    for(int i = 0; i < launches; ++i)
+        hipLaunchKernelGGL(bench_mfma_burn, dim3(cus), dim3(256), 0, nullptr, stamps, sink, iters);
+    HIP_CHECK(hipEventRecord(e1, nullptr));
+    HIP_CHECK(hipEventSynchronize(e1));
+    float ms = 0;
+    HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    std::vector<unsigned long long> h(static_cast<size_t>(waves) * 4);
+    HIP_CHECK(hipMemcpy(h.data(), stamps, h.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    std::printf("mfma_ceiling  %d CUs x 4 waves, %d v_mfma_f32_32x32x2_f32 per wave and launch, %d launches back to back\n",
+                cus, iters * 4, launches);
+    std::printf("mfma_ceiling  whole launches (event pair around all of them): %.3f ms each = %.1f TFLOP/s = %.1f %% of %.1f\n",
+                ms / launches, flop / (ms / launches) * 1e-9, flop / (ms / launches) * 1e-9 / (cus * 256 * 2.4e-3) * 100.0,
+                cus * 256 * 2.4e-3);
+    double mhz[8] = {0}, us[8] = {0};
+    int    count[8] = {0};
+    for(int w = 0; w < waves; ++w)
+    {
+        const unsigned long long* o = &h[static_cast<size_t>(w) * 4];
+        const int                 x = static_cast<int>(o[3]);
+        mhz[x] += static_cast<double>(o[2]) / static_cast<double>(o[1] - o[0]) * 100.0;
+        us[x] += static_cast<double>(o[1] - o[0]) * 0.01;
+        count[x]++;
+    }
+    double slowest = 0, mean = 0;
+    int    xcds = 0;
+    for(int x = 0; x < 8; ++x)
+        if(count[x] > 0)
+        {
+            std::printf("mfma_ceiling  XCD %d: %4d waves, shader clock %.0f MHz, loop %.1f us = %.1f %% of the matrix pipes' %d cycles\n",
+                        x, count[x], mhz[x] / count[x], us[x] / count[x],
+                        iters * 4.0 * 64.0 / (mhz[x] / count[x] * us[x] / count[x]) * 100.0, iters * 4 * 64);
+            slowest = std::max(slowest, us[x] / count[x]);
+            mean += us[x] / count[x];
+            ++xcds;
+        }
+    std::printf("mfma_ceiling  by the slowest XCD's loop: %.1f TFLOP/s; by the mean over XCDs: %.1f TFLOP/s\n",
+                flop / slowest * 1e-6, flop / (mean / xcds) * 1e-6);
+    HIP_CHECK(hipFree(stamps));
+    HIP_CHECK(hipFree(sink));
+    return 0;
 }
 
 // ---- counters: parent side ------------------------------------------------------------------------
@@ -957,6 +1067,8 @@ int main(int argc, char* argv[])
             opt.counters = true;
         else if(arg == "--host_cost")
             opt.host_cost = true;
+        else if(arg == "--mfma_ceiling")
+            opt.mfma_ceiling = true;
         else if(arg == "--uniform")
         {
             opt.uniform = true;
@@ -1007,6 +1119,10 @@ int main(int argc, char* argv[])
     if(opt.host_cost)
     {
         return run_host_cost();
+    }
+    if(opt.mfma_ceiling)
+    {
+        return run_mfma_ceiling();
     }
     if(opt.counters)
     {

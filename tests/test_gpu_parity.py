@@ -376,6 +376,28 @@ def test_bench_float_rows_parse_like_the_reference_bench():
     assert rows[8][3:] == ("384", "256", "256")
 
 
+def test_bench_float_mfma_ceiling_is_a_ceiling():
+    """--mfma_ceiling times a kernel of MFMAs only: its rate bounds every SGEMM kernel from above
+    and cannot exceed the published peak (256 CUs x 256 flop per cycle x 2.4 GHz); the per-XCD
+    lines account for all 1024 waves, each of which finds the matrix pipe busy for the whole loop."""
+    import os
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rocm_sgemm_amd",
+                       "benchmark", "bench_float")
+    _announce("bench_float --mfma_ceiling", exe)
+    out = subprocess.run([exe, "--mfma_ceiling"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    whole = re.search(r"= ([\d.]+) TFLOP/s = ([\d.]+) % of ([\d.]+)", out.stdout)
+    assert whole is not None, out.stdout
+    tflops, peak = float(whole.group(1)), float(whole.group(3))
+    assert 0.8 * peak < tflops <= 1.005 * peak, out.stdout
+    xcds = re.findall(r"XCD (\d):\s+(\d+) waves, shader clock (\d+) MHz, loop [\d.]+ us = ([\d.]+) %", out.stdout)
+    assert sum(int(x[1]) for x in xcds) == 1024 and len(xcds) == 8, out.stdout
+    for _, _, mhz, busy in xcds:
+        assert 1500 <= int(mhz) <= 2450 and 99.0 <= float(busy) <= 100.5, out.stdout
+
+
 def test_bench_float_vendor_rows_compute_the_same_product():
     """--vendor adds a rocBLAS and a hipBLASLt row under each of this library's rows; with
     --verify each vendor row carries the same sampled fp64 error figure, which pins the operand
