@@ -128,6 +128,15 @@ def shape_ok(shape):
     return True
 
 
+def sums_in_launch(shape):
+    """Whether the kernels of a tile shape can add up partial tiles themselves (the kernel's
+    tile_config::SUMS_IN_LAUNCH): at most four waves, each owning at most 64 x 64 of the macro
+    tile.  For the other shapes partial_sums makes no difference."""
+    macro_m, macro_n, _, waves_m, waves_n, _, _, waves_k = shape
+    waves = waves_m * waves_n * max(waves_k, 1)
+    return waves <= 4 and macro_m * macro_n // waves <= 64 * 64
+
+
 def swapped(shape):
     """Shape of the kernel that serves a column-major C (operands and tile swapped)."""
     macro_m, macro_n, k_tile, waves_m, waves_n, mfma, stages, waves_k = shape

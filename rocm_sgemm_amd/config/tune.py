@@ -189,6 +189,8 @@ class Tuner:
         for t in list(trials[:3]):
             if t["config"]["split_k"] == 1 and t["config"]["wave_slots"] == 1:
                 continue
+            if not space.sums_in_launch(tuple(t["config"][k] for k in space.SHAPE_KEYS)):
+                continue
             for sums in (1, 2):
                 if left <= 0:
                     break

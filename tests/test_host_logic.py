@@ -346,6 +346,11 @@ def test_space_constraints():
     assert not space.shape_ok((64, 64, 32, 1, 1, 32, 2, 4))  # one k-block per wave
     assert not space.shape_ok((256, 256, 32, 2, 4, 32, 2, 2))  # 2 x 256 x 256 floats > 160 KB
     assert space.lds_bytes(64, 64, 32, 1, 0, 2, 4) == 4 * 64 * 64 * 4  # the images, more than the stages
+    # which shapes can add up partial tiles inside the launch (at most four waves of at most 64 x 64 each)
+    assert space.sums_in_launch((128, 128, 32, 2, 2, 32, 2, 1)) and space.sums_in_launch((64, 64, 64, 1, 1, 32, 3, 4))
+    assert space.sums_in_launch((128, 64, 32, 2, 1, 32, 3, 2))
+    assert not space.sums_in_launch((256, 256, 32, 2, 2, 32, 2, 1))  # 128 x 128 per wave
+    assert not space.sums_in_launch((256, 128, 32, 4, 2, 32, 2, 1))  # eight waves
 
 
 def test_generator_outputs(tmp_path):
