@@ -23,48 +23,6 @@ struct output_scale
     }
 };
 
-// Sum of the n values fetch(0) .. fetch(n - 1), added in index order (the order every path that sums
-// partial tiles uses, so they all give the same bits).  The loads of up to eight parts are issued
-// before the first add, so a thread waits for one round trip per eight parts; indices past the end
-// are clamped to the last part, a repeated load whose value is not added.  (The kernels below are
-// bound by bandwidth all the same: eight 4 MB partials into a 4 MB output take 7 us, 5 TB/s.)
-template<int W, class V, class Fetch>
-__device__ __forceinline__ void add_parts(V& sum, int first, int n, Fetch&& fetch)
-{
-    V v[W];
-#pragma unroll
-    for(int u = 0; u < W; ++u)
-        v[u] = fetch(first + u < n ? first + u : n - 1);
-#pragma unroll
-    for(int u = 0; u < W; ++u)
-        if(first + u < n) sum += v[u];
-}
-
-template<class V, class Fetch>
-__device__ __forceinline__ V ordered_sum(int n, Fetch&& fetch)
-{
-    V sum = fetch(0);
-    for(int k = 1; k < n;)
-    {
-        if(n - k > 4)
-        {
-            add_parts<8>(sum, k, n, fetch);
-            k += 8;
-        }
-        else if(n - k > 1)
-        {
-            add_parts<4>(sum, k, n, fetch);
-            k += 4;
-        }
-        else
-        {
-            sum += fetch(k);
-            k += 1;
-        }
-    }
-    return sum;
-}
-
 // Sums the split_k partial products of batch blockIdx.y in slice order (fixed order => run-to-run
 // deterministic).  Partials are packed rows x cols matrices, [batch][slice]; the output has row
 // stride ldp and batch stride stride_p.
@@ -84,14 +42,19 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float* __restrict__ 
     for(size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < count;
         idx += stride)
     {
-        const float s = ordered_sum<float>(split_k, [&](int k) { return part[static_cast<size_t>(k) * count + idx]; });
+        float s = part[idx];
+        for(int k = 1; k < split_k; ++k)
+        {
+            s += part[static_cast<size_t>(k) * count + idx];
+        }
         float* dst = ldp == cols ? out + idx : out + (idx / cols) * ldp + idx % cols;
         *dst       = scale(s, dst);
     }
 }
 
 // Same sum, four adjacent elements per thread with 128-bit accesses: for outputs whose rows are
-// 16-byte aligned (cols, ldp and stride_p multiples of 4, aligned base).
+// 16-byte aligned (cols, ldp and stride_p multiples of 4, aligned base).  The loads of up to eight
+// slices are issued before the first add, so a thread has eight 16-byte requests in flight.
 __global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(float* __restrict__ P,
                                                                  const float* __restrict__ partial,
                                                                  int          rows,
@@ -110,9 +73,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(float* __restri
     for(size_t q = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; q < quads; q += stride)
     {
         const size_t idx = q * 4;
-        const f32x4 s = ordered_sum<f32x4>(split_k, [&](int k) {
-            return *reinterpret_cast<const f32x4*>(part + static_cast<size_t>(k) * count + idx);
-        });
+        f32x4        s   = *reinterpret_cast<const f32x4*>(part + idx);
+        int          k   = 1;
+        for(; k + 8 <= split_k; k += 8)
+        {
+            f32x4 v[8];
+#pragma unroll
+            for(int u = 0; u < 8; ++u)
+                v[u] = *reinterpret_cast<const f32x4*>(part + static_cast<size_t>(k + u) * count + idx);
+#pragma unroll
+            for(int u = 0; u < 8; ++u)
+                s += v[u]; // slice order, as in the scalar kernel
+        }
+        for(; k < split_k; ++k)
+        {
+            s += *reinterpret_cast<const f32x4*>(part + static_cast<size_t>(k) * count + idx);
+        }
         float* dst = out + (idx / cols) * ldp + idx % cols;
         f32x4  o;
         o.x = scale(s.x, dst);
@@ -155,12 +131,14 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(float* __restrict__ P,
     for(int q = blockIdx.y * blockDim.x + threadIdx.x; q < quads; q += gridDim.y * blockDim.x)
     {
         const int i = (q * 4) / bn, j = (q * 4) % bn;
-        const f32x4 s = ordered_sum<f32x4>(g_last - g_first + 1, [&](int n) {
-            const int    g    = g_first + n;
+        f32x4     s = {0.0f, 0.0f, 0.0f, 0.0f};
+        for(int g = g_first; g <= g_last; ++g)
+        {
             const int    seg  = (g * per) / k_tiles == u ? 0 : 1;
             const float* part = partial + (static_cast<size_t>(g) * 2 + seg) * tile;
-            return *reinterpret_cast<const f32x4*>(part + static_cast<size_t>(q) * 4);
-        });
+            const f32x4  v    = *reinterpret_cast<const f32x4*>(part + static_cast<size_t>(q) * 4);
+            s                 = g == g_first ? v : s + v;
+        }
         const int row = m0 + i, col = n0 + j;
         if(row < rows)
         {
