@@ -53,8 +53,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float* __restrict__ 
 }
 
 // Same sum, four adjacent elements per thread with 128-bit accesses: for outputs whose rows are
-// 16-byte aligned (cols, ldp and stride_p multiples of 4, aligned base).  The loads of up to eight
-// slices are issued before the first add, so a thread has eight 16-byte requests in flight.
+// 16-byte aligned (cols, ldp and stride_p multiples of 4, aligned base).  With nine slices or
+// more the loads of eight are issued before the first add; with fewer the plain loop is as fast
+// (eight 4 MB partials into a 4 MB output: 7.3 us = 5 TB/s, bound by bandwidth; a variant that
+// batched the loads for every slice count measured 8.2 us).
 __global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(float* __restrict__ P,
                                                                  const float* __restrict__ partial,
                                                                  int          rows,
