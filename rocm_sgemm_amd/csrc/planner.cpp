@@ -195,48 +195,48 @@ bool tail_applies(const rocm_sgemm_config& c, long long tiles, long long k_tiles
 // LDS (small tiles are bound by that: a 64 x 64 tile needs 16 bytes per 256 flop); the stream-K tail
 // or the K split add their second pass; every launch a fixed cost.  The constants are a
 // least-squares fit (log time, weighted towards each problem's fastest configs) to tuner sweeps of
-// the whole family over 68 problems between 255^3 and 5120^3, regular and ragged, on MI355X;
-// choosing each problem's config by this model lands within 2.5 % of its fastest on average
-// (1.6 - 3.7 % on held-out thirds).  Used to choose among candidate configs for problems that are not table entries, so
+// the whole family over 79 problems between 192 x 192 x 8192 and 7052 x 2436 x 856, regular and
+// ragged, on MI355X; choosing each problem's config by this model lands within 4.7 % of its fastest
+// on average (4.2 - 6.5 % on held-out thirds).  Used to choose among candidate configs for problems that are not table entries, so
 // mainly the ordering matters.
 double predict_us(const rocm_sgemm_config& c, size_t m, size_t n, size_t k, size_t batch)
 {
     const int    waves     = c.waves_m * c.waves_n * (c.waves_k > 1 ? c.waves_k : 1);
     const int    per_cu    = waves >= 4 ? 1 : 4 / (waves < 1 ? 1 : waves);
     const double wave_area = static_cast<double>(c.macro_m / c.waves_m) * (c.macro_n / c.waves_n);
-    double       eff = wave_area >= 8192 ? 0.996 : wave_area >= 4096 ? 0.970 : wave_area >= 2048 ? 0.954 : 0.926;
-    if(c.k_tile >= 64) eff *= 0.966;
-    if(c.mfma == 16) eff *= 0.950;
-    if(c.stages == 0) eff *= 0.929;
-    if(c.stages >= 3) eff *= 0.973;
+    double       eff = wave_area >= 8192 ? 1.000 : wave_area >= 4096 ? 0.953 : wave_area >= 2048 ? 0.970 : 0.921;
+    if(c.k_tile >= 64) eff *= 0.951;
+    if(c.mfma == 16) eff *= 0.947;
+    if(c.stages == 0) eff *= 0.911;
+    if(c.stages >= 3) eff *= 0.955;
     // ragged problems run the masked kernels: 16-byte loads when every dimension is a multiple
     // of 4, 4-byte loads otherwise
     const bool aligned = m % 4 == 0 && n % 4 == 0 && k % 4 == 0;
     const bool full    = m % c.macro_m == 0 && n % c.macro_n == 0 && k % c.k_tile == 0;
     if(!aligned)
-        eff *= 0.905;
+        eff *= 0.892;
     else if(!full)
-        eff *= 0.938;
+        eff *= 0.922;
     // the products of a batch are one launch: their tiles fill the waves together
     const long long tiles   = static_cast<long long>((m + c.macro_m - 1) / c.macro_m) * ((n + c.macro_n - 1) / c.macro_n)
                               * static_cast<long long>(batch);
     const long long k_tiles = static_cast<long long>((k + c.k_tile - 1) / c.k_tile);
     const double    kd      = static_cast<double>(k);
     const double    compute = 2.0 * c.macro_m * c.macro_n * kd / (614.5e3 * eff); // one CU's matrix pipes
-    // L2 -> LDS: 18.1 TB/s over the CUs; 10.7 TB/s for the 4-byte loads of a direct-to-LDS shape,
+    // L2 -> LDS: 18.75 TB/s over the CUs; 11.64 TB/s for the 4-byte loads of a direct-to-LDS shape,
     // which are bound by the number of load instructions
-    const double    l2_tbs  = !aligned && c.stages != 0 ? 10.7 : 18.1;
+    const double    l2_tbs  = !aligned && c.stages != 0 ? 11.64 : 18.75;
     const double    panels  = (c.macro_m + c.macro_n) * kd * 4.0 / (l2_tbs * 1.0e6 / model_cus);
     const double    tile_us = std::sqrt(std::sqrt(compute * compute * compute * compute + panels * panels * panels * panels)) * per_cu;
     const double    out_mb  = static_cast<double>(m) * n * 4.0 / 1.0e6 * static_cast<double>(batch);
-    double          t       = 5.5; // launch, first loads, last stores
+    double          t       = 5.86; // launch, first loads, last stores
     if(c.split_k > 1)
     {
         const long long split  = c.split_k < k_tiles ? c.split_k : k_tiles;
         const long long groups = tiles * split;
         const long long slots  = model_cus * per_cu;
         t += static_cast<double>((groups + slots - 1) / slots) * tile_us / split;
-        t += 2.5 + (split + 1) * out_mb / 4.24; // second pass: launch gap, partials at ~4.2 TB/s
+        t += 2.82 + (split + 1) * out_mb / 3.68; // second pass: launch gap, partials at ~3.7 TB/s
         return t;
     }
     long long slots = 0, r = 0;
@@ -247,8 +247,8 @@ double predict_us(const rocm_sgemm_config& c, size_t m, size_t n, size_t k, size
         if(tail)
         {
             const double tile_mb = c.macro_m * c.macro_n * 4.0 / 1.0e6;
-            // second pass: launch gap, the segments at ~7.4 TB/s (they are still in cache)
-            t += tile_us * static_cast<double>(r) / slots + 8.2 + (2.0 * slots + r) * tile_mb / 7.36;
+            // second pass: launch gap, the segments at ~5.6 TB/s
+            t += tile_us * static_cast<double>(r) / slots + 5.72 + (2.0 * slots + r) * tile_mb / 5.57;
         }
         else
         {
