@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Builds librocm_sgemm.so (gfx950), the tuner trial binary and bench_float with hipcc, in-tree.
+"""Builds librocm_sgemm.so (gfx950), the tuner trial binary, bench_float and kernel_phases with hipcc, in-tree.
 
 Plays the role of the reference's CMake targets `rocm_sgemm` and `tuner`
 (reference rocm_sgemm/CMakeLists.txt:11-89): run the config generator, compile one translation
@@ -27,6 +27,8 @@ LIB_PATH = os.path.join(PKG_DIR, "librocm_sgemm.so")
 TUNER_PATH = os.path.join(PKG_DIR, "config", "tuner")
 BENCH_SRC = os.path.join(PKG_DIR, "benchmark", "bench_float.cpp")
 BENCH_PATH = os.path.join(PKG_DIR, "benchmark", "bench_float")
+PHASES_SRC = os.path.join(PKG_DIR, "benchmark", "kernel_phases.hip")
+PHASES_PATH = os.path.join(PKG_DIR, "benchmark", "kernel_phases")
 CALLER_SRC = os.path.join(REPO_DIR, "tests", "cxx", "reference_style_caller.cpp")
 CALLER_PATH = os.path.join(REPO_DIR, "tests", "cxx", "reference_style_caller")
 # a caller that includes the reference's own host headers by path: built only where that tree is
@@ -200,6 +202,15 @@ def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR):
             raise RuntimeError("bench_float failed to build:\n" + (proc.stdout + proc.stderr)[-4000:])
         if verbose:
             print(f"linked {BENCH_PATH}")
+        # per-workgroup time stamps of a launch: its own instantiations of the kernels, compiled with
+        # the stamps switched on (the library is built without them); links nothing of the library
+        cmd = [hipcc()] + COMMON_FLAGS + ["-DROCM_SGEMM_PHASE_STAMPS", "-I", os.path.join(PKG_DIR, "csrc"),
+                                          "-x", "hip", PHASES_SRC, "-o", PHASES_PATH]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError("kernel_phases failed to build:\n" + (proc.stdout + proc.stderr)[-4000:])
+        if verbose:
+            print(f"linked {PHASES_PATH}")
     return LIB_PATH
 
 

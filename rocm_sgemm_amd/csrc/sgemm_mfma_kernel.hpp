@@ -110,6 +110,13 @@ struct gemm_args
     // ends; the wave that completes a counter adds up the tile's parts and stores the result.
     // Null: the partial tiles are left for a second kernel.
     unsigned* counters;
+#if defined(ROCM_SGEMM_PHASE_STAMPS)
+    // Only in the build of benchmark/kernel_phases (never in the library): eight 64-bit words per
+    // wave of the launch - wall clock (100 MHz) at the start of the kernel, after the prologue,
+    // after the main loop of the last segment and after the last store has completed; shader-clock
+    // cycles spent in that main loop; the XCD the wave ran on.
+    unsigned long long* stamps;
+#endif
 };
 
 template<int BM_, int BN_, int BK_, int WM_, int WN_, int MI_, bool X_KC_, bool Y_KC_, bool EDGE_, int NS_ = 0,
@@ -602,6 +609,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
         nseg    = (run1 - 1) / k_tiles > tail_u0 ? 2 : 1;
     }
 
+#if defined(ROCM_SGEMM_PHASE_STAMPS)
+    const unsigned long long stamp_start = wall_clock64();
+    unsigned long long       stamp_loop_begin = 0, stamp_loop_end = 0, stamp_cycles = 0;
+#endif
     const int batch             = blockIdx.y;
     const float* __restrict__ X = args.X + batch * args.stride_x;
     const float* __restrict__ Y = args.Y + batch * args.stride_y;
@@ -835,6 +846,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
         __syncthreads();
     }
     impl::static_for<0, NRX + NRY>([&](auto q) { read_item(decltype(q)::value, 0, 0, 0); });
+#if defined(ROCM_SGEMM_PHASE_STAMPS)
+    stamp_loop_begin = wall_clock64();
+    stamp_cycles     = clock64();
+#endif
 
     // Main loop: one barrier per K-tile, and a software pipeline written out slot by slot.
     //
@@ -925,6 +940,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
         });
         cur = nxt;
     }
+#if defined(ROCM_SGEMM_PHASE_STAMPS)
+    stamp_loop_end = wall_clock64();
+    stamp_cycles   = clock64() - stamp_cycles;
+#endif
     if constexpr(DTL)
     {
         // the clamped loads of the last iterations still target this workgroup's LDS
@@ -1302,6 +1321,20 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
         __syncthreads();
     }
     } // segments
+#if defined(ROCM_SGEMM_PHASE_STAMPS) && defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_s_waitcnt(0); // the stores have completed
+    if(args.stamps != nullptr && lane == 0)
+    {
+        unsigned long long* out
+            = args.stamps + ((static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * (NT / 64) + wave) * 8;
+        out[0] = stamp_start;
+        out[1] = stamp_loop_begin;
+        out[2] = stamp_loop_end;
+        out[3] = wall_clock64();
+        out[4] = stamp_cycles;
+        out[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20) & 7; // XCC_ID
+    }
+#endif
 }
 
 } // namespace kernel

@@ -398,6 +398,35 @@ def test_bench_float_mfma_ceiling_is_a_ceiling():
         assert 1500 <= int(mhz) <= 2450 and 99.0 <= float(busy) <= 100.5, out.stdout
 
 
+def test_kernel_phases_accounts_for_a_launch():
+    """kernel_phases instantiates the GEMM kernels with time stamps switched on (the library is
+    built without them) and prints where a launch's time goes.  The phases of a workgroup must add
+    up to its life, every workgroup must appear under one of the eight XCDs, and the main loop can
+    be no shorter than its MFMAs."""
+    import os
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rocm_sgemm_amd",
+                       "benchmark", "kernel_phases")
+    _announce("kernel_phases 2048 1024", exe)
+    out = subprocess.run([exe, "2048", "1024"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    blocks = out.stdout.strip().split("\n\n")
+    assert len(blocks) == 2, out.stdout
+    for block, groups in zip(blocks, (256, 512)):
+        rows = re.findall(r"^\s+(\d)\s+(\d+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+(\d+) MHz",
+                          block, re.M)
+        assert len(rows) == 8 and sum(int(r[1]) for r in rows) == groups, block
+        for _, _, start, prologue, loop, epilogue, end, end_max, mhz in rows:
+            total = float(start) + float(prologue) + float(loop) + float(epilogue)
+            assert abs(total - float(end)) <= 0.05 and float(end_max) >= float(end) - 0.01, block
+            assert 1500 <= int(mhz) <= 2450, block
+        busy = re.search(r"pipe busy ([\d.]+) % of the loop", block)
+        assert busy is not None and 50.0 <= float(busy.group(1)) <= 100.5, block
+        each = re.search(r"back to back: ([\d.]+) us each = ([\d.]+) TFLOP/s", block)
+        assert each is not None and 40.0 < float(each.group(2)) < 157.3, block
+
+
 def test_bench_float_vendor_rows_compute_the_same_product():
     """--vendor adds a rocBLAS and a hipBLASLt row under each of this library's rows; with
     --verify each vendor row carries the same sampled fp64 error figure, which pins the operand
