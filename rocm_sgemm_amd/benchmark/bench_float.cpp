@@ -36,6 +36,8 @@
 //                       rocm_sgemm_find_config, and per enqueued call while the GPU has queue space
 //   --mfma_ceiling      what the matrix pipes reach with nothing else to do: a kernel of MFMAs only,
 //                       one workgroup per CU, with the shader clock of every XCD during the run
+//   --l2_to_lds         bytes per cycle and CU that direct-to-LDS loads deliver from windows that fit
+//                       the L2s and from windows that do not
 //   --pmc               short run for use under rocprofv3 --pmc: 2 warm-up + 5 timed launches and
 //                       one plain 64 MiB copy kernel, whose known traffic calibrates the
 //                       FETCH_SIZE / WRITE_SIZE counters
@@ -106,6 +108,7 @@ struct options
     bool             vendor      = false;
     bool             pmc         = false; // child mode under rocprofv3
     bool             counters    = false; // parent mode: collect counters row by row
+    bool             l2_to_lds    = false; // time the L2 -> LDS path alone instead of the timing table
     bool             mfma_ceiling = false; // time the matrix pipes alone instead of the timing table
     bool             host_cost   = false; // host-side cost of a call instead of the timing table
     std::vector<int> layouts; // bit 2 = A col, bit 1 = B col, bit 0 = C col; empty = all eight
@@ -190,6 +193,7 @@ void print_usage(const char* program)
               << "  --host_cost        host microseconds per call: planning alone, and enqueueing plain / split-K /\n"
               << "                     stream-K-tail products, one shape repeated and several shapes in turn\n"
               << "  --mfma_ceiling     TFLOP/s of a kernel that issues MFMAs only, and the shader clock of every XCD meanwhile\n"
+              << "  --l2_to_lds        bytes per cycle and CU of direct-to-LDS loads from L2-resident and larger windows\n"
               << "  --help             Show this help message\n"
               << "\nExamples:\n"
               << "  " << program << " --shapes 512:1024:2048\n"
@@ -474,6 +478,83 @@ int run_mfma_ceiling()
                 flop / slowest * 1e-6, flop / (mean / xcds) * 1e-6);
     HIP_CHECK(hipFree(stamps));
     HIP_CHECK(hipFree(sink));
+    return 0;
+}
+
+// ---- the path from L2 into LDS alone ----------------------------------------------------------------
+// Every workgroup (256 threads, one per CU) streams 16-byte pieces straight into LDS
+// (buffer_load_dwordx4 ... lds, the instruction the GEMM kernels move their operands with) from a
+// window of its own that it reads over and over: a window larger than the CU's vector cache and
+// small enough for all windows to stay in the L2s measures L2 -> LDS; a larger one measures what
+// comes from beyond the L2.  The figure bounds the operand traffic a GEMM kernel can ask of a CU.
+template<int WINDOW_KB>
+__global__ __launch_bounds__(256) void bench_l2_to_lds(const float* __restrict__ src, float* __restrict__ sink,
+                                                       unsigned long long* __restrict__ cycles, int iters)
+{
+    __shared__ __attribute__((aligned(16))) float lds[4 * 1024]; // 16 KB: four loads of the workgroup
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float* base = src + static_cast<size_t>(blockIdx.x) * WINDOW_KB * 256;
+    const __amdgpu_buffer_rsrc_t rsrc
+        = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, WINDOW_KB * 1024, 0x00020000);
+    const int                wave = threadIdx.x / 64;
+    const unsigned long long c0   = clock64();
+    for(int i = 0; i < iters; ++i)
+    {
+#pragma unroll
+        for(int u = 0; u < 4; ++u) // 4 KB per load of the workgroup
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(lds + (u * 256 + wave * 64) * 4),
+                                                     16, threadIdx.x * 16, ((i * 4 + u) % (WINDOW_KB / 4)) * 4096, 0, 0);
+        if((i & 7) == 7) __builtin_amdgcn_s_waitcnt(0x0070 | 8); // at most eight loads of the wave in flight
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    const unsigned long long c1 = clock64();
+    if(lds[threadIdx.x] == 0.12345f) sink[0] = lds[threadIdx.x];
+    if(threadIdx.x == 0) cycles[blockIdx.x] = c1 - c0;
+#else
+    (void)src, (void)sink, (void)cycles, (void)iters, (void)lds;
+#endif
+}
+
+template<int WINDOW_KB>
+int run_l2_to_lds_case(int groups, const float* src, float* sink, unsigned long long* cycles)
+{
+    const int iters = 4000; // 64 MB per workgroup
+    for(int r = 0; r < 3; ++r)
+        hipLaunchKernelGGL(bench_l2_to_lds<WINDOW_KB>, dim3(groups), dim3(256), 0, nullptr, src, sink, cycles, iters);
+    HIP_CHECK(hipDeviceSynchronize());
+    std::vector<unsigned long long> h(groups);
+    HIP_CHECK(hipMemcpy(h.data(), cycles, groups * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    double mean = 0;
+    for(unsigned long long v : h)
+        mean += static_cast<double>(v);
+    mean /= groups;
+    const double per_cu = iters * 16384.0 / mean;
+    std::printf("l2_to_lds  window %4d KB per workgroup, %3d workgroups (%5.1f MB in all): %5.1f bytes per cycle and CU = %5.1f TB/s at 2.4 GHz\n",
+                WINDOW_KB, groups, groups * WINDOW_KB / 1024.0, per_cu, per_cu * groups * 2.4e-3);
+    return 0;
+}
+
+int run_l2_to_lds()
+{
+    float *            src, *sink;
+    unsigned long long* cycles;
+    HIP_CHECK(hipMalloc(&src, 256u << 20));
+    HIP_CHECK(hipMemset(src, 0, 256u << 20));
+    HIP_CHECK(hipMalloc(&sink, sizeof(float)));
+    HIP_CHECK(hipMalloc(&cycles, 1024 * sizeof(unsigned long long)));
+    hipDeviceProp_t prop;
+    HIP_CHECK(hipGetDeviceProperties(&prop, 0));
+    const int cus = prop.multiProcessorCount;
+    for(int groups : {cus / 4, cus})
+    {
+        run_l2_to_lds_case<64>(groups, src, sink, cycles);
+        run_l2_to_lds_case<128>(groups, src, sink, cycles);
+        run_l2_to_lds_case<256>(groups, src, sink, cycles);
+        run_l2_to_lds_case<1024>(groups, src, sink, cycles);
+    }
+    HIP_CHECK(hipFree(src));
+    HIP_CHECK(hipFree(sink));
+    HIP_CHECK(hipFree(cycles));
     return 0;
 }
 
@@ -1069,6 +1150,8 @@ int main(int argc, char* argv[])
             opt.host_cost = true;
         else if(arg == "--mfma_ceiling")
             opt.mfma_ceiling = true;
+        else if(arg == "--l2_to_lds")
+            opt.l2_to_lds = true;
         else if(arg == "--uniform")
         {
             opt.uniform = true;
@@ -1123,6 +1206,10 @@ int main(int argc, char* argv[])
     if(opt.mfma_ceiling)
     {
         return run_mfma_ceiling();
+    }
+    if(opt.l2_to_lds)
+    {
+        return run_l2_to_lds();
     }
     if(opt.counters)
     {

@@ -427,6 +427,26 @@ def test_kernel_phases_accounts_for_a_launch():
         assert each is not None and 40.0 < float(each.group(2)) < 157.3, block
 
 
+def test_bench_float_l2_to_lds_probe():
+    """--l2_to_lds streams direct-to-LDS loads from windows that fit the L2s and from windows that
+    do not: a CU cannot take more than 64 bytes per cycle, and what comes from beyond the L2 is
+    slower than what comes from it."""
+    import os
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rocm_sgemm_amd",
+                       "benchmark", "bench_float")
+    _announce("bench_float --l2_to_lds", exe)
+    out = subprocess.run([exe, "--l2_to_lds"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    rows = re.findall(r"window\s+(\d+) KB per workgroup,\s+(\d+) workgroups .*?:\s+([\d.]+) bytes per cycle and CU", out.stdout)
+    assert len(rows) == 8, out.stdout
+    rate = {(int(w), int(g)): float(r) for w, g, r in rows}
+    assert all(1.0 < r <= 64.5 for r in rate.values()), out.stdout
+    groups = max(g for _, g in rate)
+    assert rate[(1024, groups)] < rate[(64, groups)], out.stdout
+
+
 def test_bench_float_vendor_rows_compute_the_same_product():
     """--vendor adds a rocBLAS and a hipBLASLt row under each of this library's rows; with
     --verify each vendor row carries the same sampled fp64 error figure, which pins the operand
