@@ -163,6 +163,7 @@ _BASE_SHAPES = [
     # K-tiles of 64: half as many pipeline steps (barriers, waits) per unit of depth, which is
     # what small tiles with few MFMAs per step are short of
     (128, 128, 64, 2, 2, 32, 2, 1),
+    (128, 128, 64, 4, 2, 32, 2, 1),  # eight waves: 1 % over the four-wave form at 2048^3 (141.0 against 139.6 TFLOP/s)
     (64, 64, 64, 2, 2, 32, 2, 1),
     # v_mfma_f32_16x16x4_f32: a 128-bit LDS read is fully used even by narrow wave tiles
     (128, 128, 32, 2, 2, 16, 3, 1),
