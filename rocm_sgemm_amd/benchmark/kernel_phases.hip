@@ -165,22 +165,32 @@ int run_case(const char* title, int M, int N, int K, int group_m, int split)
     quantiles(v_start, "start"), quantiles(v_pro, "prologue"), quantiles(v_loop, "loop");
     quantiles(v_epi, "epilogue"), quantiles(v_end, "end");
     std::printf("  end of the main loop, spread over the waves of a workgroup: mean %.2f, max %.2f\n", skew_sum / grid, skew_max);
-    // MFMA cycles of one wave's main loop, and how many waves share a SIMD on average (workgroups
-    // beyond what LDS lets a CU hold wait for a free CU instead)
+    // MFMA cycles of one wave's main loop against the cycles it spent there, and - because waves that
+    // share a SIMD take turns at its matrix pipe in no fixed pattern (a loop without stalls lets the
+    // older wave run ahead and the younger one wait) - the share of all matrix-pipe cycles of the GPU
+    // that MFMAs fill between the first wave entering its main loop and the last one leaving it.
     const double mfma_cycles = static_cast<double>(Cfg::TM * Cfg::TN) * (Cfg::MI == 32 ? 64.0 : 32.0)
                                * (static_cast<double>(K) / split) / (Cfg::MI == 32 ? 2.0 : 4.0) / Cfg::WK;
     int          cus = 256;
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, 0);
-    const double resident_groups = std::min<double>(160.0 * 1024 / Cfg::LDS_BYTES >= 1.0 ? static_cast<int>(160 * 1024 / Cfg::LDS_BYTES) : 1,
-                                                    static_cast<double>(grid) / cus);
-    const double waves_per_simd  = std::max(1.0, resident_groups * waves / 4.0);
-    double       loop_cycles     = 0;
-    for(unsigned g = 0; g < grid; ++g)
-        loop_cycles += static_cast<double>(st[static_cast<size_t>(g) * waves * 8 + 4]);
-    loop_cycles /= grid;
-    std::printf("  main loop: %.0f shader cycles per wave on average; its MFMAs occupy the matrix pipe for %.0f; "
-                "%.2f waves share a SIMD: pipe busy %.1f %% of the loop\n",
-                loop_cycles, mfma_cycles, waves_per_simd, mfma_cycles * waves_per_simd / loop_cycles * 100.0);
+    double             loop_cycles = 0, mhz = 0;
+    unsigned long long loop_first = ~0ull, loop_last = 0;
+    for(size_t w = 0; w < static_cast<size_t>(grid) * waves; ++w)
+    {
+        const unsigned long long* o = &st[w * 8];
+        loop_cycles += static_cast<double>(o[4]);
+        loop_first = std::min(loop_first, o[1]);
+        loop_last  = std::max(loop_last, o[2]);
+        mhz += o[2] > o[1] ? static_cast<double>(o[4]) / static_cast<double>(o[2] - o[1]) * 100.0 : 0.0;
+    }
+    loop_cycles /= static_cast<double>(grid) * waves;
+    mhz /= static_cast<double>(grid) * waves;
+    const double span_us    = (loop_last - loop_first) * 0.01;
+    const double pipe_total = 4.0 * cus * span_us * mhz; // matrix-pipe cycles of the GPU in that span
+    std::printf("  main loop: %.0f shader cycles per wave on average, %.0f of them its own MFMAs; from the first wave "
+                "entering its loop to the last leaving (%.2f us at %.0f MHz): pipe busy %.1f %% of the loop\n",
+                loop_cycles, mfma_cycles, span_us, mhz,
+                mfma_cycles * static_cast<double>(grid) * waves / pipe_total * 100.0);
     CHECK(hipFree(A));
     CHECK(hipFree(B));
     CHECK(hipFree(C));

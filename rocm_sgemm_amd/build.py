@@ -79,7 +79,8 @@ def _compile(job):
 
 
 def _check_no_spills(log, src):
-    """A kernel that spills registers to scratch memory is a bug in the tile-shape constraints."""
+    """A kernel that spills registers to scratch memory is a bug in the tile-shape constraints.
+    Returns one line per spilling kernel."""
     bad = []
     name = None
     for line in log.splitlines():
@@ -89,8 +90,7 @@ def _check_no_spills(log, src):
             n = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
             if n != 0:
                 bad.append((name, n))
-    if bad:
-        raise RuntimeError(f"{os.path.basename(src)}: kernels use scratch memory (spills): {bad}")
+    return [f"{os.path.basename(src)}: {name} spills {n} bytes per lane" for name, n in bad]
 
 
 def build(jobs=None, force=False, tuner=True, verbose=True, defines=(), lib_path=None,
@@ -131,6 +131,7 @@ def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR):
 
     jobs = jobs or min(16, os.cpu_count() or 4)
     failed = []
+    spilling = []
     done = 0
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         for src, rc, log, cached in pool.map(_compile, work):
@@ -138,14 +139,19 @@ def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR):
             if rc != 0:
                 failed.append((src, log))
                 continue
-            if not cached and not os.environ.get("RSG_ALLOW_SPILLS"):
-                _check_no_spills(log, src)
+            if not cached:
+                spilling += _check_no_spills(log, src)
             if verbose and not cached:
                 print(f"[{done}/{len(work)}] compiled {os.path.basename(src)}", flush=True)
     if failed:
         for src, log in failed:
             sys.stderr.write(f"--- {src}\n{log}\n")
         raise RuntimeError(f"{len(failed)} translation units failed to compile")
+    if spilling and not os.environ.get("RSG_ALLOW_SPILLS"):
+        for obj in (w[1] for w in work):  # nothing that spills stays cached as good
+            if any(os.path.basename(obj)[:-2] in line for line in spilling) and os.path.exists(obj + ".stamp"):
+                os.remove(obj + ".stamp")
+        raise RuntimeError("kernels use scratch memory (register spills):\n  " + "\n  ".join(spilling))
 
     objs = [w[1] for w in work]
     link = [hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB_PATH] + objs

@@ -147,43 +147,26 @@ def swapped(shape):
 # the valid points of PARAM_SPACE: big tiles for the compute-bound squares, small ones so that
 # skinny or small problems still produce >= 256 workgroups.
 _BASE_SHAPES = [
-    # direct-to-LDS (stages >= 2); small tiles get deeper rings, their K-tiles being short
+    # direct-to-LDS (stages >= 2); four waves, one per SIMD, each with the whole register file
     (256, 256, 32, 2, 2, 32, 2, 1),
-    (256, 256, 32, 2, 4, 32, 2, 1),
     (256, 128, 32, 2, 2, 32, 2, 1),
-    (256, 128, 32, 2, 2, 32, 3, 1),
-    (256, 128, 32, 4, 2, 32, 2, 1),
     (128, 128, 32, 2, 2, 32, 2, 1),
-    (128, 128, 32, 2, 2, 32, 3, 1),
-    (128, 128, 32, 2, 2, 32, 4, 1),
     (128, 64, 32, 2, 2, 32, 3, 1),
     (64, 64, 32, 2, 2, 32, 2, 1),
-    (64, 64, 32, 2, 2, 32, 4, 1),
-    (32, 32, 32, 1, 1, 32, 4, 1),
-    # K-tiles of 64: half as many pipeline steps (barriers, waits) per unit of depth, which is
-    # what small tiles with few MFMAs per step are short of
+    # eight waves: two per SIMD cover each other's stalls in prologue and epilogue
+    (256, 128, 32, 4, 2, 32, 2, 1),
+    (128, 128, 64, 4, 2, 32, 2, 1),
+    # K-tiles of 64: half as many pipeline steps (barriers, waits) per unit of depth
     (128, 128, 64, 2, 2, 32, 2, 1),
-    (128, 128, 64, 4, 2, 32, 2, 1),  # eight waves: 1 % over the four-wave form at 2048^3 (141.0 against 139.6 TFLOP/s)
     (64, 64, 64, 2, 2, 32, 2, 1),
-    # v_mfma_f32_16x16x4_f32: a 128-bit LDS read is fully used even by narrow wave tiles
-    (128, 128, 32, 2, 2, 16, 3, 1),
-    (64, 64, 32, 2, 2, 16, 3, 1),
-    (32, 32, 32, 1, 1, 16, 4, 1),
     # waves along K: small macro tiles whose waves still own a 64 x 64 (or 64 x 32) wave tile, for
     # problems that need many tiles to fill the GPU
     (64, 64, 64, 1, 1, 32, 3, 4),
     (64, 32, 64, 1, 1, 32, 3, 4),
     (128, 64, 32, 2, 1, 32, 3, 2),
     (64, 64, 128, 1, 1, 32, 2, 4),
-    # register-staged (stages = 0): K-tiles of 16 for very shallow problems, the one-wave tiles
-    # for one-row or one-column problems, and the classic double-buffered 128 x 128 and 64 x 64
-    # tiles as the tuner's point of comparison
+    # register-staged (stages = 0): K-tiles of 16 for very shallow problems
     (256, 128, 16, 2, 2, 32, 0, 1),
-    (128, 128, 16, 2, 2, 32, 0, 1),
-    (128, 128, 32, 2, 2, 32, 0, 1),
-    (64, 64, 32, 2, 2, 32, 0, 1),
-    (32, 32, 32, 1, 1, 32, 0, 1),
-    (32, 32, 32, 1, 1, 16, 0, 1),
 ]
 
 

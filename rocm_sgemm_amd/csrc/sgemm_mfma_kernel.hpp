@@ -190,10 +190,13 @@ struct tile_config
     // workgroup per CU; a K-split kernel whose LDS lets two workgroups share a CU (128 x 64 and
     // 64 x 128 with WK = 2) then takes 264 - 270 registers for the summing code of the epilogue,
     // just over the 256 that two waves per SIMD leave each, and loses 5 % (2048^3: 131.6 against
-    // 137.8 TFLOP/s).  Only those kernels are bounded; the others fit as they are.
+    // 137.8 TFLOP/s).  The same goes for the other kernels whose waves hold 64 accumulator
+    // registers (128 x 128 on 2 x 2 waves: the masked variants take 260 - 264 registers unbounded).
     static constexpr int WG_PER_CU_BY_LDS = 160 * 1024 / LDS_BYTES;
     static constexpr int MIN_WAVES_PER_SIMD
-        = WK > 1 && WG_PER_CU_BY_LDS >= 2 && BM * BN / (WM * WN) >= 64 * 64 ? 2 * ((NT / 64 + 3) / 4) : 1;
+        = WG_PER_CU_BY_LDS >= 2 && ((WK > 1 && BM * BN / (WM * WN) >= 64 * 64) || BM * BN / (WM * WN * WK) == 64 * 64)
+              ? 2 * ((NT / 64 + 3) / 4)
+              : 1;
 
     // Swizzle of a depth-contiguous direct-to-LDS image: rows of BK floats, CPR 16-byte chunks
     // each, RPL rows per 64-bank line.
@@ -645,8 +648,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
     // register-staged path: thread-fixed offsets, staging registers, range-checked loads
     using map_x              = impl::chunk_map<X_KC, BM, BK, NT>;
     using map_y              = impl::chunk_map<Y_KC, BN, BK, NT>;
-    const int          x_voff = DTL ? 0 : map_x::thread_offset(tid, ldx);
-    const int          y_voff = DTL ? 0 : map_y::thread_offset(tid, ldy);
+    // Everything below that depends on the lane (offsets into the operands, LDS addresses) is set
+    // up by lane_setup() at the start of every segment, from a copy of the thread index that the
+    // compiler cannot see through: computed once ahead of the segment loop, those registers would
+    // stay occupied through the epilogue, which needs every register it can get.
+    int tid_s = tid, h_s = h, c_s = c;
+    int x_voff = 0, y_voff = 0;
     const float* const x_end  = X + args.extent_x;
     const float* const y_end  = Y + args.extent_y;
     auto               bytes_to = [](const float* from, const float* end) -> unsigned {
@@ -671,18 +678,21 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
             }
         }
     };
-    auto store_item = [&](int i, int buf, int t) { // staging register i (K-tile t) -> LDS stage buf
+    // `ragged_c`: the K-tile may be the last one of a depth that is not a multiple of BK, so what lies
+    // beyond K is masked; a std::false_type caller guarantees a whole K-tile and pays for no masks
+    auto store_item = [&](int i, int buf, int t, auto ragged_c) { // staging register i (K-tile t) -> LDS stage buf
         if constexpr(!DTL)
         {
-            float*    sx    = lds + buf * Cfg::STAGE;
-            const int k_rem = k_end - (k_begin + t * BK);
+            constexpr bool masked = EDGE && decltype(ragged_c)::value;
+            float*         sx     = lds + buf * Cfg::STAGE;
+            const int      k_rem  = k_end - (k_begin + t * BK);
             if(i < CX)
                 impl::store_chunk<X_KC, BM, BK, Cfg::LDX, NT>(
-                    i, sx, impl::mask_chunk<X_KC, EDGE, BM, BK, NT>(stage_x[i], k_rem, tid), tid);
+                    i, sx, impl::mask_chunk<X_KC, masked, BM, BK, NT>(stage_x[i], k_rem, tid_s), tid_s);
             else
                 impl::store_chunk<Y_KC, BN, BK, Cfg::LDY, NT>(
                     i - CX, sx + Cfg::X_SIZE,
-                    impl::mask_chunk<Y_KC, EDGE, BN, BK, NT>(stage_y[i - CX], k_rem, tid), tid);
+                    impl::mask_chunk<Y_KC, masked, BN, BK, NT>(stage_y[i - CX], k_rem, tid_s), tid_s);
         }
     };
 
@@ -705,25 +715,17 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
     // check itself.
     int x_dpos[DTL && EDGE && X_KC ? NVX : 1];
     int y_dpos[DTL && EDGE && Y_KC ? NVY : 1];
-    if constexpr(DTL)
-    {
-        impl::static_for<0, NVX>([&](auto i) { x_doff[decltype(i)::value] = dma_x::lane_offset(decltype(i)::value, tid, ldx); });
-        impl::static_for<0, NVY>([&](auto i) { y_doff[decltype(i)::value] = dma_y::lane_offset(decltype(i)::value, tid, ldy); });
-        if constexpr(EDGE && X_KC)
-            impl::static_for<0, NVX>([&](auto i) { x_dpos[decltype(i)::value] = dma_x::depth_pos(decltype(i)::value, tid); });
-        if constexpr(EDGE && Y_KC)
-            impl::static_for<0, NVY>([&](auto i) { y_dpos[decltype(i)::value] = dma_y::depth_pos(decltype(i)::value, tid); });
-    }
-    auto dma_item = [&](int i, int t, int buf) { // HBM -> LDS stage buf, piece i of K-tile t
+    auto dma_item = [&](int i, int t, int buf, auto ragged_c) { // HBM -> LDS stage buf, piece i of K-tile t
         if constexpr(DTL)
         {
-            float*    st    = lds + buf * Cfg::STAGE;
-            const int k_rem = k_end - (k_begin + t * BK); // depth left from this K-tile's origin
+            constexpr bool masked = EDGE && decltype(ragged_c)::value; // see store_item
+            float*         st     = lds + buf * Cfg::STAGE;
+            const int      k_rem  = k_end - (k_begin + t * BK); // depth left from this K-tile's origin
             if(i < CX)
             {
                 int       voff = x_doff[i % NVX];
                 const int soff = i * dma_x::STEP * ldx;
-                if constexpr(EDGE && X_KC)
+                if constexpr(masked && X_KC)
                     voff = x_dpos[i % NVX] < k_rem ? voff : impl::dma_reject;
                 const float* tile = x_tile(t);
                 impl::dma_load<DGX>(tile, EDGE ? min(bytes_to(tile, x_end), impl::dma_max_bytes) : 0x7FFFFFFFu,
@@ -734,7 +736,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
                 const int j    = i - CX;
                 int       voff = y_doff[j % NVY];
                 const int soff = j * dma_y::STEP * ldy;
-                if constexpr(EDGE && Y_KC)
+                if constexpr(masked && Y_KC)
                     voff = y_dpos[j % NVY] < k_rem ? voff : impl::dma_reject;
                 const float* tile = y_tile(t);
                 impl::dma_load<DGY>(tile, EDGE ? min(bytes_to(tile, y_end), impl::dma_max_bytes) : 0x7FFFFFFFu,
@@ -748,20 +750,42 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
     constexpr int KBC = 64 / MI; // 16-byte chunks of a row per k-block and lane group
     int           xs_base[DTL && X_KC ? NKB : 1];
     int           ys_base[DTL && Y_KC ? NKB : 1];
-    if constexpr(DTL && X_KC)
-    {
-        const int u = h ^ dma_x::swz(c);
-        impl::static_for<0, NKB>([&](auto kb) {
-            xs_base[decltype(kb)::value] = (wm0 + c) * BK + ((((kb0 + decltype(kb)::value) * KBC) ^ u) * 4);
-        });
-    }
-    if constexpr(DTL && Y_KC)
-    {
-        const int u = h ^ dma_y::swz(c);
-        impl::static_for<0, NKB>([&](auto kb) {
-            ys_base[decltype(kb)::value] = (wn0 + c) * BK + ((((kb0 + decltype(kb)::value) * KBC) ^ u) * 4);
-        });
-    }
+    auto lane_setup = [&]() {
+#if defined(__HIP_DEVICE_COMPILE__)
+        tid_s = tid;
+        asm volatile("" : "+v"(tid_s));
+#endif
+        h_s = (tid_s % 64) / MI;
+        c_s = (tid_s % 64) % MI;
+        if constexpr(!DTL)
+        {
+            x_voff = map_x::thread_offset(tid_s, ldx);
+            y_voff = map_y::thread_offset(tid_s, ldy);
+        }
+        else
+        {
+            impl::static_for<0, NVX>([&](auto i) { x_doff[decltype(i)::value] = dma_x::lane_offset(decltype(i)::value, tid_s, ldx); });
+            impl::static_for<0, NVY>([&](auto i) { y_doff[decltype(i)::value] = dma_y::lane_offset(decltype(i)::value, tid_s, ldy); });
+            if constexpr(EDGE && X_KC)
+                impl::static_for<0, NVX>([&](auto i) { x_dpos[decltype(i)::value] = dma_x::depth_pos(decltype(i)::value, tid_s); });
+            if constexpr(EDGE && Y_KC)
+                impl::static_for<0, NVY>([&](auto i) { y_dpos[decltype(i)::value] = dma_y::depth_pos(decltype(i)::value, tid_s); });
+        }
+        if constexpr(DTL && X_KC)
+        {
+            const int u = h_s ^ dma_x::swz(c_s);
+            impl::static_for<0, NKB>([&](auto kb) {
+                xs_base[decltype(kb)::value] = (wm0 + c_s) * BK + ((((kb0 + decltype(kb)::value) * KBC) ^ u) * 4);
+            });
+        }
+        if constexpr(DTL && Y_KC)
+        {
+            const int u = h_s ^ dma_y::swz(c_s);
+            impl::static_for<0, NKB>([&](auto kb) {
+                ys_base[decltype(kb)::value] = (wn0 + c_s) * BK + ((((kb0 + decltype(kb)::value) * KBC) ^ u) * 4);
+            });
+        }
+    };
     float fx[2][TM][4];
     float fy[2][TN][4];
     // depth offset of this wave's k-blocks inside an image that is not addressed through the
@@ -771,14 +795,15 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
     auto  read_item = [&](int q, int slot, int buf, int kb) { // LDS stage buf -> fragment set slot
         const float* sx = lds + buf * Cfg::STAGE;
         if(q < NRX)
-            impl::read_one<X_KC, DTL, TM, VM, Cfg::LDX, MI>(q, fx[slot], sx + x_koff, xs_base, wm0, kb, h, c);
+            impl::read_one<X_KC, DTL, TM, VM, Cfg::LDX, MI>(q, fx[slot], sx + x_koff, xs_base, wm0, kb, h_s, c_s);
         else
             impl::read_one<Y_KC, DTL, TN, VN, Cfg::LDY, MI>(q - NRX, fy[slot], sx + Cfg::X_SIZE + y_koff,
-                                                            ys_base, wn0, kb, h, c);
+                                                            ys_base, wn0, kb, h_s, c_s);
     };
 
     for(int seg = 0; seg < nseg; ++seg)
     {
+    lane_setup();
     if(tail)
     {
         const int u = tail_u0 + seg;
@@ -814,13 +839,21 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
     ntiles  = (k_end - k_begin + BK - 1) / BK;
     x_panel = X + (X_KC ? static_cast<size_t>(m0) * ldx : static_cast<size_t>(m0));
     y_panel = Y + (Y_KC ? static_cast<size_t>(n0) * ldy : static_cast<size_t>(n0));
+    // The accumulators start at zero: each tile is cleared by one MFMA of zeros onto the constant
+    // 0 (0 * 0 + 0), which lands in the accumulation registers directly.  From a plain `= 0.0f`
+    // the compiler sometimes builds a vector of zeros in ordinary registers, keeps it across the
+    // segment loop and spills it.
+    {
+        float nothing = 0.0f;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "+v"(nothing)); // one register holding 0.0f, not a constant the compiler can see through
+#endif
 #pragma unroll
-    for(int i = 0; i < TM; ++i)
+        for(int i = 0; i < TM; ++i)
 #pragma unroll
-        for(int j = 0; j < TN; ++j)
-#pragma unroll
-            for(int v = 0; v < ACC; ++v)
-                acc[i][j][v] = 0.0f;
+            for(int j = 0; j < TN; ++j)
+                acc[i][j] = impl::mfma<MI>(nothing, nothing, acc_t{});
+    }
 
     // Prologue.  Tile indices past the end are clamped to the last tile (a redundant, in-bounds
     // load whose data is never used), which keeps the main loop free of branches.
@@ -830,22 +863,32 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
     // loads that may still be in flight when a tile is needed: those of the NS - 2 tiles after it
     // (the wait counter holds 6 bits: a deeper ring than that waits for more than it must)
     constexpr int IN_FLIGHT = DTL ? ((NS - 2) * (CX + CY) < 64 ? (NS - 2) * (CX + CY) : 63) : 0;
+    // K-tile t sits in stage (first_stage + t) % NS, with first_stage chosen so that the K-tiles
+    // left after the first ntiles % NS of them start in stage 0 (see the main loop).
+    const int peeled      = ntiles % NS;
+    const int first_stage = peeled == 0 ? 0 : NS - peeled;
+    auto      stage_after = [](int stage, int n) { // (stage + n) % NS for 0 <= n < NS
+        const int u = stage + n;
+        return u >= NS ? u - NS : u;
+    };
     if constexpr(DTL)
     {
         impl::static_for<0, NS - 1>([&](auto s_c) {
-            constexpr int s = decltype(s_c)::value;
-            impl::static_for<0, CX + CY>([&](auto i) { dma_item(decltype(i)::value, min(s, last_tile), s); });
+            constexpr int s     = decltype(s_c)::value;
+            const int     stage = stage_after(first_stage, s);
+            impl::static_for<0, CX + CY>(
+                [&](auto i) { dma_item(decltype(i)::value, min(s, last_tile), stage, std::true_type{}); });
         });
         impl::ring_barrier<IN_FLIGHT>();
     }
     else
     {
         impl::static_for<0, CX + CY>([&](auto i) { load_item(decltype(i)::value, 0); });
-        impl::static_for<0, CX + CY>([&](auto i) { store_item(decltype(i)::value, 0, 0); });
+        impl::static_for<0, CX + CY>([&](auto i) { store_item(decltype(i)::value, first_stage, 0, std::true_type{}); });
         impl::static_for<0, CX + CY>([&](auto i) { load_item(decltype(i)::value, min(1, last_tile)); });
         __syncthreads();
     }
-    impl::static_for<0, NRX + NRY>([&](auto q) { read_item(decltype(q)::value, 0, 0, 0); });
+    impl::static_for<0, NRX + NRY>([&](auto q) { read_item(decltype(q)::value, 0, first_stage, 0); });
 #if defined(ROCM_SGEMM_PHASE_STAMPS)
     stamp_loop_begin = wall_clock64();
     stamp_cycles     = clock64();
@@ -883,12 +926,15 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
                                  : (DTL && (DGX == 1 || DGY == 1)) ? (NS >= 3 || DENSE_KBS > NKB - 1 ? NKB - 1 : DENSE_KBS)
                                                     : 1;
     constexpr int MOVE_SLOTS   = MOVE_KBS * SLOTS;
-    int           cur          = 0; // stage of K-tile t
-    for(int t = 0; t < ntiles; ++t)
-    {
-        const int nxt        = cur == NS - 1 ? 0 : cur + 1; // stage of K-tile t + 1
-        const int fill_stage = cur == 0 ? NS - 1 : cur - 1; // stage of K-tile t + NS - 1
-        const int fill_tile  = min(t + (DTL ? NS - 1 : 2), last_tile);
+    // One K-tile of the pipeline: K-tile t sits in stage `cur_c`.  With `ragged_c` false the caller
+    // guarantees that every K-tile touched here (t + 1, and the one being fetched) is a whole one
+    // before the last, so nothing is clamped or masked.
+    auto k_tile_step = [&](int t, auto cur_c, auto ragged_c) {
+        constexpr bool ragged     = decltype(ragged_c)::value;
+        const int      cur        = cur_c; // stage of K-tile t
+        const int      nxt        = cur == NS - 1 ? 0 : cur + 1; // stage of K-tile t + 1
+        const int      fill_stage = cur == 0 ? NS - 1 : cur - 1; // stage of K-tile t + NS - 1
+        const int      fill_tile  = ragged ? min(t + (DTL ? NS - 1 : 2), last_tile) : t + (DTL ? NS - 1 : 2);
         impl::static_for<0, NKB>([&](auto kb_c) {
             constexpr int  kb       = decltype(kb_c)::value;
             constexpr int  slot     = kb & 1;
@@ -927,9 +973,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
                     impl::static_for<gb, ge>([&](auto g_c) {
                         constexpr int g = decltype(g_c)::value;
                         if constexpr(DTL)
-                            dma_item(g, fill_tile, fill_stage);
+                            dma_item(g, fill_tile, fill_stage, ragged_c);
                         else if constexpr(g % 2 == 0)
-                            store_item(g / 2, nxt, t + 1);
+                            store_item(g / 2, nxt, t + 1, ragged_c);
                         else
                             load_item(g / 2, fill_tile);
                     });
@@ -938,7 +984,61 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
-        cur = nxt;
+    };
+    // Keeps the accumulators in the accumulation registers across the boundaries between the loops
+    // below (an empty asm with a register-class constraint: no instruction).  Without it the
+    // register allocator moves accumulators to ordinary registers and back at those boundaries.
+    auto pin_acc = [&]() { // not a generic lambda: the asm operand must name `acc` directly
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+        for(int i = 0; i < TM; ++i)
+#pragma unroll
+            for(int j = 0; j < TN; ++j)
+                asm volatile("" : "+a"(acc[i][j]));
+#endif
+    };
+    // Steady state: NS K-tiles per trip, so that every stage index is a constant.  The LDS address
+    // of every fragment read and the LDS target of every load are then loop-invariant (a register
+    // set up once, plus an immediate offset) and the loop holds no vector-ALU instruction at all.
+    // That matters more than it looks: on this part a vector-ALU instruction issued into a stream
+    // of back-to-back MFMAs holds up the next MFMA by about 13 cycles (scalar instructions, LDS
+    // reads, direct-to-LDS loads and barriers cost nothing there), and a loop that computes
+    // `stage offset + lane offset` for its reads spends six of them per K-tile.
+    // The ntiles % NS K-tiles that do not fill a trip come first, one at a time with the stage in
+    // a register; the prologue has placed K-tile 0 so that the first whole trip starts in stage 0.
+    pin_acc();
+    {
+        int stage = first_stage;
+        for(int t = 0; t < peeled; ++t)
+        {
+            k_tile_step(t, stage, std::true_type{});
+            stage = stage_after(stage, 1);
+        }
+    }
+    pin_acc();
+    if constexpr(!EDGE)
+    {
+        // nothing to mask; the clamp of the tile index is one scalar instruction per K-tile
+        for(int t = peeled; t < ntiles; t += NS)
+        {
+            impl::static_for<0, NS>([&](auto s_c) { k_tile_step(t + decltype(s_c)::value, s_c, std::true_type{}); });
+        }
+    }
+    else
+    {
+        // Only the last trip touches the last K-tile (it fetches it, or multiplies it): the trips
+        // before it run without the masks of a ragged depth, whose compares and selects are
+        // vector-ALU instructions, two per load.
+        int t = peeled;
+        for(; t + 2 * NS <= ntiles; t += NS)
+        {
+            impl::static_for<0, NS>([&](auto s_c) { k_tile_step(t + decltype(s_c)::value, s_c, std::false_type{}); });
+        }
+        pin_acc();
+        if(t < ntiles)
+        {
+            impl::static_for<0, NS>([&](auto s_c) { k_tile_step(t + decltype(s_c)::value, s_c, std::true_type{}); });
+        }
     }
 #if defined(ROCM_SGEMM_PHASE_STAMPS)
     stamp_loop_end = wall_clock64();
@@ -1039,15 +1139,32 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
             }
             else
             {
-#pragma unroll
-                for(int j = 0; j < TN; ++j)
-                {
-                    const int col = t.col0 + wn0 + impl::tile_index<Y_KC, VN, MI>(j, c_e);
-                    if(!EDGE || col < t.col_end)
+                // one column per tile: tile j of this lane is column MI * j + c of the wave tile
+                static_assert(impl::tile_index<Y_KC, VN, MI>(1, 0) == MI || TN == 1, "tiles are stacked here");
+                float* const pcol = prow + (t.col0 + wn0 + c_e);
+                impl::static_for<0, TN>([&](auto j_c) {
+                    constexpr int j = decltype(j_c)::value;
+                    if(!EDGE || t.col0 + wn0 + c_e + MI * j < t.col_end)
                     {
-                        prow[col] = vals[j][v];
+#if defined(__HIP_DEVICE_COMPILE__)
+                        if constexpr(std::is_same_v<std::remove_reference_t<decltype(vals)>, acc_t[TN]>)
+                        {
+                            // straight from the accumulation register: left to itself the compiler
+                            // may first copy all accumulators of the wave into ordinary registers
+                            // (operands are locals of this lambda: an asm statement in a generic
+                            // lambda cannot name what it captures)
+                            float* const where = pcol;
+                            const float  what  = vals[j][v];
+                            asm volatile("global_store_dword %0, %1, off offset:%2" ::"v"(where), "a"(what), "n"(MI * j * 4)
+                                         : "memory");
+                        }
+                        else
+#endif
+                        {
+                            pcol[MI * j] = vals[j][v];
+                        }
                     }
-                }
+                });
             }
         }
     };
@@ -1164,10 +1281,18 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
         if constexpr(WK > 1)
             put_summed(t);
         else
+        {
+#if defined(__HIP_DEVICE_COMPILE__)
+            // put_row may store accumulation registers through asm statements, whose operands the
+            // compiler's hazard recogniser does not see: a store must not read a register within 18
+            // wait states of the MFMA that wrote it.  Volatile asm statements keep their order.
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#endif
             impl::static_for<0, TM>([&](auto i_c) {
                 put_row(t, decltype(i_c)::value, acc[decltype(i_c)::value], std::integral_constant<int, 0>{},
                         std::integral_constant<int, ACC>{});
             });
+        }
     };
     auto share_tile = [&](const tile_place& t) {
         if constexpr(WK > 1)
@@ -1273,12 +1398,18 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
         // knows that every other part is complete in memory, adds them all up in a fixed order -
         // K slices in slice order, tail segments in workgroup order - and stores the result.  No
         // wave ever waits for another.
-        // Ordering.  Writers: the parts are stored with the agent-scope cache policy; the fence makes
-        // the wave wait until those stores are complete (and keeps the compiler from moving them)
-        // before the ticket is drawn.  Reader: the parts are read with the same policy by loads
-        // issued after the ticket has come back, so no cache can hand out a line that is older than
-        // the ticket.
+        // Ordering.  Writers: the parts are stored with the agent-scope cache policy (written through,
+        // never left dirty in this XCD's L2), and the wave then waits until every one of those
+        // stores has been acknowledged (s_waitcnt vmcnt(0): on this target stores count in vmcnt
+        // like loads) before it draws the ticket.  A wave's stores and its atomic go to different
+        // memory channels and are ordered at issue only, so without that wait the ticket could
+        // become visible before a part has landed.  The workgroup-scope fences emit no
+        // instruction here; they only keep the compiler from moving memory accesses across the
+        // ticket.  Reader: the parts are read with the same cache policy by loads that are issued
+        // after the ticket has come back (the branch below depends on its value), so no cache can
+        // hand out a line that is older than the ticket.
         share_tile(mine);
+        impl::wait_all_loads();
         const int tile_id  = tail ? tail_u0 + seg : wg; // tail: number of the tail tile; else the tile
         const int expected = tail ? min(((tile_id + 1) * k_tiles - 1) / args.tail_per, args.tail_groups - 1)
                                         - (tile_id * k_tiles) / args.tail_per + 1

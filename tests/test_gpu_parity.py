@@ -780,7 +780,7 @@ def test_strided_batched_with_explicit_configs_split_k_and_broadcast():
     rng = np.random.default_rng(77)
     fams = {tuple(f.as_dict()[k] for k in ("macro_m", "macro_n", "k_tile", "stages")): f.as_dict()
             for f in rs.family()}
-    for key, split in (((128, 128, 32, 2), 1), ((128, 128, 32, 2), 3), ((64, 64, 32, 0), 2),
+    for key, split in (((128, 128, 32, 2), 1), ((128, 128, 32, 2), 3), ((256, 128, 16, 0), 2),
                        ((256, 256, 32, 2), 1)):
         cfg = dict(fams[key], split_k=split, group_m=2, wave_slots=0)
         for (la, lb, lc) in ((0, 0, 0), (1, 0, 1), (0, 1, 0)):
