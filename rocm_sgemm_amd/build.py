@@ -94,25 +94,38 @@ def _check_no_spills(log, src):
 
 
 def build(jobs=None, force=False, tuner=True, verbose=True, defines=(), lib_path=None,
-          obj_dir=None):
+          obj_dir=None, out_dir=None, shapes=None):
     """Generates, compiles and links.  `defines` (extra -D macros), `lib_path` and `obj_dir` exist
-    so that an experimental variant can be built beside the shipped library."""
+    so that an experimental variant can be built beside the shipped library.  `out_dir` builds a
+    whole side tree instead - generated sources, objects, `librocm_sgemm.so` and `config/tuner`
+    under that directory - for the tuner's exploration mode, which compiles tile shapes from
+    outside the shipped family (config/space.py: explore()) without touching the shipped library;
+    only the library and the trial binary are built there, and `shapes` limits the side library
+    to those tile shapes (plus the default config's)."""
     sys.path.insert(0, os.path.join(PKG_DIR, "config"))
     import generate_config  # noqa: E402
 
-    global COMMON_FLAGS
-    base_flags = COMMON_FLAGS
-    COMMON_FLAGS = base_flags + [f"-D{d}" for d in defines]
+    global COMMON_FLAGS, GEN_DIR, TUNER_PATH
+    base = (COMMON_FLAGS, GEN_DIR, TUNER_PATH)
+    if out_dir is not None:
+        out_dir = os.path.abspath(out_dir)
+        GEN_DIR = os.path.join(out_dir, "gen")
+        TUNER_PATH = os.path.join(out_dir, "config", "tuner")
+        os.makedirs(os.path.dirname(TUNER_PATH), exist_ok=True)
+        lib_path = os.path.join(out_dir, "librocm_sgemm.so")
+        obj_dir = os.path.join(out_dir, "obj")
+        COMMON_FLAGS = [GEN_DIR if f == base[1] else f for f in COMMON_FLAGS]
+    COMMON_FLAGS = COMMON_FLAGS + [f"-D{d}" for d in defines]
     try:
         return _build(generate_config, jobs, force, tuner, verbose, lib_path or LIB_PATH,
-                      obj_dir or OBJ_DIR)
+                      obj_dir or OBJ_DIR, side_tree=out_dir is not None, shapes=shapes)
     finally:
-        COMMON_FLAGS = base_flags
+        COMMON_FLAGS, GEN_DIR, TUNER_PATH = base
 
 
-def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR):
+def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR, side_tree=False, shapes=None):
     os.makedirs(OBJ_DIR, exist_ok=True)
-    kernel_sources = generate_config.generate(CONFIG_JSON, GEN_DIR)
+    kernel_sources = generate_config.generate(CONFIG_JSON, GEN_DIR, shapes)
     host_sources = [os.path.join(CSRC, "dispatch.cpp"), os.path.join(CSRC, "planner.cpp"),
                     os.path.join(CSRC, "api.cpp")]
     headers = [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith(".hpp")]
@@ -163,13 +176,15 @@ def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR):
 
     if tuner:
         cmd = [hipcc()] + COMMON_FLAGS + ["-x", "hip", os.path.join(PKG_DIR, "config", "tuner.cpp"),
-                                          "-o", TUNER_PATH, "-L", PKG_DIR, "-lrocm_sgemm",
+                                          "-o", TUNER_PATH, "-L", os.path.dirname(LIB_PATH), "-lrocm_sgemm",
                                           "-Wl,-rpath,$ORIGIN/.."]
         proc = subprocess.run(cmd, capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError("tuner build failed:\n" + (proc.stdout + proc.stderr)[-4000:])
         if verbose:
             print(f"linked {TUNER_PATH}")
+        if side_tree:
+            return LIB_PATH
         # a program written against the reference's public header, linked against this library
         cmd = [hipcc(), "-std=c++17", "-O2", f"--offload-arch={ARCH}", "-Wno-unused-command-line-argument",
                "-I", os.path.join(REPO_DIR, "include"), "-x", "hip", CALLER_SRC, "-o", CALLER_PATH,
@@ -228,7 +243,19 @@ def main():
     ap.add_argument("--define", action="append", default=[], help="extra -D macro (experiments)")
     ap.add_argument("--lib-path", default=None, help="where to link the library (experiments)")
     ap.add_argument("--obj-dir", default=None, help="object directory (experiments)")
+    ap.add_argument("--explore", nargs="+", metavar="SHAPE", default=None,
+                    help="build a side library of these tile shapes (macro_m,macro_n,k_tile,waves_m,waves_n,"
+                         "mfma,stages,waves_k each) and its trial binary under --explore-dir, for "
+                         "`config/tune.py --explore ... --explore-prebuilt`; the shipped library is not touched")
+    ap.add_argument("--explore-dir", default=os.path.join(PKG_DIR, "_build", "explore"))
     a = ap.parse_args()
+    if a.explore:
+        sys.path.insert(0, os.path.join(PKG_DIR, "config"))
+        import space  # noqa: E402
+        shapes = space.explore([tuple(int(x) for x in s.split(",")) for s in a.explore])
+        build(jobs=a.jobs, force=a.force, out_dir=a.explore_dir, shapes=shapes)
+        print(f"side library of {len(shapes)} tile shapes in {a.explore_dir}")
+        return
     build(jobs=a.jobs, force=a.force, tuner=not a.no_tuner, defines=a.define, lib_path=a.lib_path,
           obj_dir=a.obj_dir)
 

@@ -156,6 +156,10 @@ _BASE_SHAPES = [
     # eight waves: two per SIMD cover each other's stalls in prologue and epilogue
     (256, 128, 32, 4, 2, 32, 2, 1),
     (128, 128, 64, 4, 2, 32, 2, 1),
+    # K-tile of 16 in a direct-to-LDS ring: 48 KB of LDS and 128 accumulators, so two workgroups
+    # share a CU and one's prologue and epilogue hide behind the other's main loop.  Found by the
+    # tuner's exploration mode (8192 x 8192 x 1024: 1.5 % over the best shape of the family then)
+    (256, 128, 16, 2, 2, 32, 2, 1),
     # K-tiles of 64: half as many pipeline steps (barriers, waits) per unit of depth
     (128, 128, 64, 2, 2, 32, 2, 1),
     (64, 64, 64, 2, 2, 32, 2, 1),
@@ -171,20 +175,61 @@ _BASE_SHAPES = [
 
 
 _FAMILY = None
+_EXTRA_SHAPES = []
+
+
+def _closed(shapes):
+    out = []
+    for s in shapes:
+        for t in (tuple(s), swapped(tuple(s))):
+            if not shape_ok(t):
+                raise ValueError(f"tile shape {t} violates the kernel's constraints")
+            if t not in out:
+                out.append(t)
+    return out
 
 
 def family():
+    """Tile shapes compiled into the library, plus (exploration only) those of explore()."""
     global _FAMILY
     if _FAMILY is None:
-        out = []
-        for s in _BASE_SHAPES:
-            for t in (s, swapped(s)):
-                if not shape_ok(t):
-                    raise ValueError(f"tile shape {t} violates the kernel's constraints")
-                if t not in out:
-                    out.append(t)
-        _FAMILY = out
+        _FAMILY = _closed(_BASE_SHAPES)
+    return list(_FAMILY) + [s for s in _EXTRA_SHAPES if s not in _FAMILY]
+
+
+def shipped_family():
+    """The family without exploration shapes."""
+    family()
     return list(_FAMILY)
+
+
+def explore(shapes):
+    """Adds tile shapes from outside the shipped family for this process: the generator then emits
+    kernels for them (into a side library, see build.build(out_dir=...)) and the tuner times them.
+    Returns the shapes added (closed under `swapped`)."""
+    global _EXTRA_SHAPES
+    _EXTRA_SHAPES = [s for s in _closed(shapes) if s not in shipped_family()]
+    return list(_EXTRA_SHAPES)
+
+
+def neighbours(shape):
+    """Valid tile shapes one step away from `shape` in the search space (another K-tile, ring depth,
+    wave grid or waves along K on the same macro tile; the macro tile halved or doubled along one
+    side), for the tuner's exploration mode."""
+    bm, bn, bk, wm, wn, mfma, stages, wk = shape
+    out = set()
+    for k in PARAM_SPACE["k_tile"]:
+        for st in PARAM_SPACE["stages"]:
+            out.add((bm, bn, k, wm, wn, mfma, st, wk))
+    for a in PARAM_SPACE["waves_m"]:
+        for b in PARAM_SPACE["waves_n"]:
+            for w in PARAM_SPACE["waves_k"]:
+                out.add((bm, bn, bk, a, b, mfma, stages, w))
+    for m2, n2 in ((bm * 2, bn), (bm, bn * 2), (bm // 2, bn), (bm, bn // 2)):
+        if m2 in PARAM_SPACE["macro_m"] and n2 in PARAM_SPACE["macro_n"]:
+            out.add((m2, n2, bk, wm, wn, mfma, stages, wk))
+    out.discard(tuple(shape))
+    return sorted(s for s in out if shape_ok(s))
 
 
 def all_valid_shapes():

@@ -17,11 +17,20 @@ What differs, because the kernels do:
     phases 3 and 4 try the best configs without the stream-K tail and with the partial tiles summed
     inside the launch / by a second kernel.
     `--budget` caps the number of trials per (size, layout) as in the reference.
+  * `--explore` leaves the precompiled family, which is what the reference's tuner does for every
+    trial (it compiles any valid point of its space through hipRTC, reference tuner.cpp:183-216,
+    234-383, tune.py:163-232): tile shapes from outside the family - given on the command line, or
+    the neighbours in the search space of the family's three fastest shapes for each problem - are
+    compiled into a side library (build.build(out_dir=...), a minute for a dozen shapes), timed by a
+    trial binary linked against it, and compared with the family's best.  A shape that wins is
+    reported; it joins the library by being added to space._BASE_SHAPES.
 
 usage examples
   python tune.py                                   # 1024..8192 cubes, all 8 layouts
   python tune.py --sizes 4096,4096,4096 --layouts r,r,r c,c,c
   python tune.py --input gemm_config.json --sizes 128,4096,4096 --output gemm_config_tuned.json
+  python tune.py --explore --sizes 2048,2048,2048 --layouts r,r,r          # neighbours of the best shapes
+  python tune.py --explore 256,128,16,2,2,32,2,1 128,128,16,2,2,32,4,1 --sizes 8192,8192,8192 --layouts r,r,r
 """
 
 import argparse
@@ -84,7 +93,7 @@ def split_candidates(shape, M, N, K):
 
 class Tuner:
     def __init__(self, tuner_bin, budget=150, iters=20, max_memory=space.LDS_BYTES_PER_CU, seed=42,
-                 runner=subprocess.run, verbose=True):
+                 runner=subprocess.run, verbose=True, shapes=None):
         self.tuner_bin = tuner_bin
         self.budget = budget
         self.iters = iters
@@ -92,7 +101,8 @@ class Tuner:
         self.seed = seed  # the search is exhaustive and deterministic; kept for CLI compatibility
         self.runner = runner
         self.verbose = verbose
-        self.shapes = [s for s in space.family()
+        # the tile shapes the trial binary's library holds (its sweep times all of them)
+        self.shapes = [s for s in (space.family() if shapes is None else shapes)
                        if space.max_lds_bytes(s[0], s[1], s[2]) <= max_memory]
 
     def log(self, *a):
@@ -207,7 +217,13 @@ class Tuner:
         shape = tuple(best["config"][k] for k in space.SHAPE_KEYS)
         self.log(f"  best {best['config']}  {best['avg_ms']:.4f} ms "
                  f"({2.0 * M * N * K / best['avg_ms'] * 1e-9:.1f} TFLOP/s, {len(trials)} trials)")
+        by_shape = {}
+        for t in trials:  # fastest trial of every tile shape, fastest shape first
+            key = tuple(t["config"][k] for k in space.SHAPE_KEYS)
+            if key not in by_shape or t["avg_ms"] < by_shape[key]:
+                by_shape[key] = t["avg_ms"]
         return {"M": M, "N": N, "K": K, "layout": layout, "config": best["config"],
+                "shape_ranking": sorted(by_shape.items(), key=lambda kv: kv[1]),
                 "avg_time_ms": best["avg_ms"], "evaluations": len(trials),
                 "memory_used_bytes": space.max_lds_bytes(*shape[:3], shape[6], shape[7]),
                 "space_coverage_percent": round(100.0 * len({tuple(t['config'][k] for k in space.SHAPE_KEYS) for t in trials}) / max(1, len(self.shapes)), 1)}
@@ -222,6 +238,90 @@ class Tuner:
                 if rec is not None:
                     results[(M, N, K) + tuple(layout)] = rec
         return results
+
+
+# -- exploration: tile shapes from outside the compiled family --------------------------------------
+
+def parse_shapes(items):
+    out = []
+    for it in items:
+        vals = tuple(int(x) for x in it.split(","))
+        if len(vals) != len(space.SHAPE_KEYS):
+            raise ValueError(f"a tile shape is {len(space.SHAPE_KEYS)} ints ({','.join(space.SHAPE_KEYS)}), got {it!r}")
+        if not space.shape_ok(vals):
+            raise ValueError(f"tile shape {vals} violates the kernel's constraints")
+        out.append(vals)
+    return out
+
+
+def default_side_build(out_dir, shapes):
+    """Compiles `shapes` (and the default config's shape) into <out_dir>/librocm_sgemm.so and links
+    <out_dir>/config/tuner against it.  Returns the path of that trial binary."""
+    sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+    from rocm_sgemm_amd import build as lib_build  # noqa: E402
+    lib_build.build(out_dir=out_dir, shapes=shapes, tuner=True, verbose=False)
+    return os.path.join(out_dir, "config", "tuner")
+
+
+def explore(sizes, layouts, shapes, family_tuner, out_dir, max_shapes=12, side_build=default_side_build,
+            make_tuner=None, log=print):
+    """Times tile shapes from outside the family against the family's best for every (size, layout).
+
+    `shapes`: the shapes to try; empty = for every problem the neighbours (space.neighbours) of the
+    family's three fastest shapes, at most `max_shapes` in all.  `family_tuner` is a Tuner on the
+    shipped trial binary; `side_build(out_dir, shapes)` builds the side library and returns its
+    trial binary; `make_tuner(path, shapes)` makes the Tuner for it (tests replace both).
+    Returns [{M, N, K, layout, family: {config, avg_ms}, explored: {config, avg_ms} | None,
+    winner: bool, shape_ranking: [...]}]."""
+    shipped = space.shipped_family()
+    family_recs = {}
+    for (M, N, K) in sizes:
+        for layout in layouts:
+            log(f"family sweep {M}x{N}x{K} A,B,C={layout}")
+            family_recs[(M, N, K) + tuple(layout)] = family_tuner.tune_problem(M, N, K, layout)
+    candidates = [s for s in shapes if s not in shipped]
+    if not candidates:
+        pool = []
+        for rec in family_recs.values():
+            if rec is None:
+                continue
+            for shape, _ in rec["shape_ranking"][:3]:
+                for n in space.neighbours(shape):
+                    if n not in shipped and n not in pool:
+                        pool.append(n)
+        # round-robin over the problems' neighbourhoods would be fairer; sorted keeps it reproducible
+        candidates = sorted(pool)[:max_shapes]
+    if not candidates:
+        log("nothing to explore: every candidate is in the family already")
+        return []
+    added = space.explore(candidates)
+    log(f"compiling {len(added)} tile shapes outside the family: {added}")
+    side_bin = side_build(out_dir, added)
+    side = make_tuner(side_bin, added) if make_tuner else Tuner(
+        side_bin, budget=family_tuner.budget, iters=family_tuner.iters, max_memory=family_tuner.max_memory,
+        runner=family_tuner.runner, verbose=family_tuner.verbose, shapes=added)
+    out = []
+    for key, fam in family_recs.items():
+        M, N, K = key[:3]
+        layout = key[3:]
+        log(f"exploring {M}x{N}x{K} A,B,C={layout}")
+        rec = side.tune_problem(M, N, K, layout)
+        # the side library also holds the default config's shape: only shapes outside the family count
+        ranking = [(s, ms) for s, ms in (rec["shape_ranking"] if rec else []) if s not in shipped]
+        best = None
+        if rec is not None and tuple(rec["config"][k] for k in space.SHAPE_KEYS) not in shipped:
+            best = {"config": rec["config"], "avg_ms": rec["avg_time_ms"]}
+        elif ranking:
+            best = {"config": dict(zip(space.SHAPE_KEYS, ranking[0][0])), "avg_ms": ranking[0][1]}
+        fam_best = {"config": fam["config"], "avg_ms": fam["avg_time_ms"]} if fam else None
+        winner = bool(best and fam_best and best["avg_ms"] < fam_best["avg_ms"])
+        if best and fam_best:
+            log(f"  family {fam_best['avg_ms']:.4f} ms, best outside {best['avg_ms']:.4f} ms "
+                f"({(fam_best['avg_ms'] / best['avg_ms'] - 1.0) * 100.0:+.1f} %): "
+                + ("the explored shape wins" if winner else "the family holds"))
+        out.append({"M": M, "N": N, "K": K, "layout": list(layout), "family": fam_best, "explored": best,
+                    "winner": winner, "shape_ranking": [[list(s), ms] for s, ms in ranking]})
+    return out
 
 
 # -- JSON in / out (schema of reference config/gemm_config.json:1-30 with the new config keys) -----
@@ -280,6 +380,15 @@ def main(argv=None):
     ap.add_argument("--iters", type=int, default=20, help="timed launches per trial")
     ap.add_argument("--tuner", default=os.path.join(HERE, "tuner"), help="trial binary")
     ap.add_argument("--output", default="gemm_config_tuned.json")
+    ap.add_argument("--explore", nargs="*", metavar="SHAPE", default=None,
+                    help="time tile shapes from outside the compiled family (" + ",".join(space.SHAPE_KEYS)
+                         + " each); without shapes: the neighbours of the family's fastest shapes")
+    ap.add_argument("--explore-dir", default=os.path.join(os.path.dirname(HERE), "_build", "explore"),
+                    help="where the side library and its trial binary are built")
+    ap.add_argument("--explore-max", type=int, default=12, help="most shapes compiled when none are named")
+    ap.add_argument("--explore-prebuilt", action="store_true",
+                    help="the side library in --explore-dir already holds the named shapes: do not compile "
+                         "(build it beforehand with `python -m rocm_sgemm_amd.build --explore SHAPE ...`)")
     args = ap.parse_args(argv)
 
     if args.gpu_arch != "gfx950":
@@ -299,6 +408,16 @@ def main(argv=None):
 
     tuner = Tuner(args.tuner, budget=args.budget, iters=args.iters, max_memory=args.max_memory,
                   seed=args.seed)
+    if args.explore is not None:
+        prebuilt = (lambda out_dir, shapes: os.path.join(out_dir, "config", "tuner")) if args.explore_prebuilt \
+            else default_side_build
+        found = explore(sizes, layouts, parse_shapes(args.explore), tuner, args.explore_dir, args.explore_max,
+                        side_build=prebuilt)
+        with open(args.output, "w") as f:
+            json.dump({"explored": found}, f, indent=4)
+        wins = [r for r in found if r["winner"]]
+        print(f"explored {len(found)} problems, {len(wins)} won by a shape outside the family; wrote {args.output}")
+        return 0
     new = tuner.tune_all(sizes, layouts, baselines_for)
     merged = merge_results(existing, new)
     with open(args.output, "w") as f:

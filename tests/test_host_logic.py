@@ -463,6 +463,64 @@ def test_tuner_budget_and_split_candidates():
     assert tune.parse_sizes(["128,4096,4096"]) == [(128, 4096, 4096)]
 
 
+def test_tuner_exploration_finds_a_planted_optimum_outside_the_family(tmp_path):
+    """--explore: the planted optimum is a tile shape the library does not ship.  The family sweep
+    cannot see it; the exploration compiles it (here: a stand-in for the side build records what it
+    was asked to compile), times it through the side trial binary and reports it as the winner."""
+    planted = (256, 128, 16, 2, 2, 32, 2, 1)
+    assert space.shape_ok(planted) and planted not in space.shipped_family()
+    assert planted in space.neighbours((256, 128, 32, 2, 2, 32, 2, 1))
+    built = []
+
+    def runner_for(which):
+        def run(cmd, capture_output=True, text=True, timeout=None):
+            # the shipped binary knows the family only, the side binary what was compiled into it
+            shapes = space.shipped_family() if which == "family" else built[-1][1]
+            if cmd[1] == "--sweep":
+                splits = [int(x) for x in cmd[cmd.index("--splits") + 1].split(",")]
+                lines = []
+                for sh in shapes:
+                    for sp in splits:
+                        ms = 0.5 if sh == planted and sp == 1 else (1.0 if sh == (256, 128, 32, 2, 2, 32, 2, 1) and sp == 1 else 2.0)
+                        lines.append("cfg " + " ".join(map(str, sh[:7] + (sp, 4, 0, sh[7], 0)))
+                                     + f" avg_ms {ms:.4f} min_ms {ms:.4f} tflops 1.00 ok 1")
+                return _FakeProc("\n".join(lines))
+            return _FakeProc("time: 3.0000 ms  min: 3.0000 ms  avg_tflops: 1  max_tflops: 1\n")
+        return run
+
+    def side_build(out_dir, shapes):
+        built.append((out_dir, list(shapes)))
+        return os.path.join(out_dir, "config", "tuner")
+
+    fam = tune.Tuner("tuner", budget=30, runner=runner_for("family"), verbose=False)
+    try:
+        found = tune.explore([(4096, 4096, 4096)], [(0, 0, 0)], [], fam, str(tmp_path), max_shapes=64,
+                             side_build=side_build,
+                             make_tuner=lambda path, shapes: tune.Tuner(path, budget=30, runner=runner_for("side"),
+                                                                        verbose=False, shapes=shapes),
+                             log=lambda *a: None)
+        assert len(built) == 1 and planted in built[0][1]
+        assert all(sh not in space.shipped_family() for sh in built[0][1])
+        assert len(found) == 1 and found[0]["winner"]
+        assert tuple(found[0]["explored"]["config"][k] for k in space.SHAPE_KEYS) == planted
+        assert found[0]["explored"]["avg_ms"] == 0.5 and found[0]["family"]["avg_ms"] == 1.0
+        # named shapes are taken as they are; one that is in the family already is not compiled again
+        built.clear()
+        found = tune.explore([(4096, 4096, 4096)], [(0, 0, 0)], [planted, (256, 256, 32, 2, 2, 32, 2, 1)], fam,
+                             str(tmp_path), side_build=side_build,
+                             make_tuner=lambda path, shapes: tune.Tuner(path, budget=30, runner=runner_for("side"),
+                                                                        verbose=False, shapes=shapes),
+                             log=lambda *a: None)
+        assert [sorted(b[1]) for b in built] == [sorted({planted, space.swapped(planted)})]
+        assert found[0]["winner"]
+    finally:
+        space.explore([])  # leave the family as shipped for the other tests
+    assert space.family() == space.shipped_family()
+    assert tune.parse_shapes(["256,128,16,2,2,32,2,1"]) == [planted]
+    with pytest.raises(ValueError):
+        tune.parse_shapes(["256,256,32,2,4,32,3,1"])  # three stages of 64 KB exceed the LDS
+
+
 # ---- a caller written against the reference's public header ---------------------------------------
 
 CALLER = os.path.join(REPO, "tests", "cxx", "reference_style_caller")
