@@ -467,7 +467,7 @@ def test_tuner_exploration_finds_a_planted_optimum_outside_the_family(tmp_path):
     """--explore: the planted optimum is a tile shape the library does not ship.  The family sweep
     cannot see it; the exploration compiles it (here: a stand-in for the side build records what it
     was asked to compile), times it through the side trial binary and reports it as the winner."""
-    planted = (256, 128, 16, 2, 2, 32, 2, 1)
+    planted = (256, 128, 16, 2, 2, 32, 4, 1)
     assert space.shape_ok(planted) and planted not in space.shipped_family()
     assert planted in space.neighbours((256, 128, 32, 2, 2, 32, 2, 1))
     built = []
@@ -516,7 +516,7 @@ def test_tuner_exploration_finds_a_planted_optimum_outside_the_family(tmp_path):
     finally:
         space.explore([])  # leave the family as shipped for the other tests
     assert space.family() == space.shipped_family()
-    assert tune.parse_shapes(["256,128,16,2,2,32,2,1"]) == [planted]
+    assert tune.parse_shapes(["256,128,16,2,2,32,4,1"]) == [planted]
     with pytest.raises(ValueError):
         tune.parse_shapes(["256,256,32,2,4,32,3,1"])  # three stages of 64 KB exceed the LDS
 
