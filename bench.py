@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """SGEMM benchmark of the MI355X library: prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps 100] [--warmup 10] [--no-layouts] [--no-cpu] [--counters]
+    python bench.py [--gpus 1] [--steps 100] [--warmup 10] [--no-layouts] [--no-cpu] [--no-counters] [--counters]
 
 Workload (the reference README's identity-multiply methodology, reference README.md:27-47):
 M = N = K = 4096, A, B, C row-major, A uniform[-1, 1) from mt19937(seed 0), B = identity; the output
@@ -14,9 +14,16 @@ back and the region is closed by one device synchronisation.
 
 Also in the line:
   roofline      MFMA-bound: achieved = 2MNK / mean launch duration, peak = 157.3 TFLOP/s (dense FP32
-                matrix peak of MI355X); traffic = HBM bytes per launch measured by --counters in this
-                run, else read from the summary an earlier --counters run left under profiles/
-                (traffic_source says which), else null
+                matrix peak of MI355X); traffic = HBM bytes per launch from rocprofv3 --pmc passes
+                of this run (four short child processes; skipped with --no-counters or where
+                rocprofv3 is missing, then read from the summary under profiles/; traffic_source
+                says which)
+  counters      from the same passes: matrix-pipe busy %, LDS bank conflicts %, HBM bytes per launch
+  dense_4096    the same 4096^3 product on uniform[-1, 1) A and B (identity B draws less power and
+                runs about 1 % faster): NN / NT / TN / TT (A, B column- or row-major in BLAS terms:
+                row-major = T) with C row-major, avg and min-time TFLOP/s each
+  held_out      shapes that are not entries of the tuned table, in mixed layouts: the config the
+                planner chose, its rate, and the vendor library's on the same operands
   layouts       the reference bench's default cubes, 1024^3 to 8192^3, in the four A/B storage
                 combinations (NN/NT/TN/TT) with C row- and column-major, uniform[-1, 1) A and B.
                 Per row: avg / min-time TFLOP/s of the per-launch event pairs, the sustained rate
@@ -30,8 +37,7 @@ Also in the line:
                 1024^3 as the reference runs it, all usable threads at 1024^3 and on a bounded
                 sample of 4096^3 (labelled extrapolated when cut), timed on this host; plus, where
                 it has been built, the reference's own GPU kernel on this GPU for context
---counters additionally runs the timed loop under rocprofv3 --pmc (MFMA busy, LDS bank conflicts,
-HBM bytes) and writes profiles/sgemm_mfma_4096_rrr_counters.txt.
+--counters also writes the counter summary to profiles/sgemm_mfma_4096_rrr_counters.txt.
 """
 
 import argparse
@@ -190,6 +196,60 @@ def bench_shapes(rs, steps, warmup):
         row["kernel_config"] = rs.find_config(m, n, k).as_dict()
         out[f"{m}x{n}x{k}"] = row
         del dA, dB, dC, a2, b2
+    return out
+
+
+# Shapes that are NOT entries of the tuned table (config/gemm_config.json must never list them):
+# (M, N, K, layout of A, B, C; 0 = row-major, 1 = column-major).  What runs is the planner's choice.
+HELD_OUT = [(3072, 5120, 2048, 0, 1, 0), (1536, 1200, 900, 1, 1, 0), (6000, 6000, 6000, 0, 0, 0),
+            (2304, 768, 12288, 1, 0, 1), (5000, 1500, 2500, 0, 0, 1), (640, 9000, 3100, 1, 0, 0)]
+
+
+def vendor_operands(dA, dB, m, n, k, la, lb, lc):
+    """torch views such that torch.matmul(x, y) is the product in the caller's storage orders: a
+    column-major C (M x N) is the row-major N x M matrix C^T = B^T A^T."""
+    a = dA.view(m, k) if la == 0 else dA.view(k, m).t()
+    b = dB.view(k, n) if lb == 0 else dB.view(n, k).t()
+    return (a, b) if lc == 0 else (b.t(), a.t())
+
+
+def bench_held_out(rs, steps, warmup):
+    import torch
+    torch.backends.cuda.matmul.allow_tf32 = False
+    names = {0: "r", 1: "c"}
+    table = {key for key, _ in rs.table()}
+    out = {}
+    stream = torch.cuda.current_stream()
+    for (m, n, k, la, lb, lc) in HELD_OUT:
+        dA, dB = uniform_device(m * k, 7), uniform_device(k * n, 8)
+        dC = torch.empty(m * n, dtype=torch.float32, device="cuda:0")
+        flop_ms = 2.0 * m * n * k / 140e9
+        n_steps = max(5, min(steps, int(200 / max(flop_ms, 0.01))))
+        row = measure(lambda: rs.gemm(dC, dA, dB, m, n, k, lc, la, lb, stream=stream), m, n, k, n_steps, warmup)
+        x, y = vendor_operands(dA, dB, m, n, k, la, lb, lc)
+        vendor = measure(lambda: torch.matmul(x, y), m, n, k, n_steps, warmup)
+        row["vendor_avg_tflops"] = vendor["avg_tflops"]
+        row["vendor_back_to_back_tflops"] = vendor["back_to_back_tflops"]
+        row["planned_config"] = rs.find_config(m, n, k, la, lb, lc).as_dict()
+        row["in_tuned_table"] = (m, n, k, la, lb, lc) in table
+        out[f"{m}x{n}x{k} {names[la]}{names[lb]}{names[lc]}"] = row
+        del dA, dB, dC, x, y
+    return out
+
+
+def bench_dense_4096(rs, steps, warmup):
+    """4096^3 on uniform operands, C row-major, the four A / B storage orders under their BLAS
+    names (a row-major operand is a transposed one: reference test/rocblas/test.cpp:4-14)."""
+    import torch
+    dA, dB = uniform_device(M * K, 1), uniform_device(K * N, 2)
+    dC = torch.empty(M * N, dtype=torch.float32, device="cuda:0")
+    stream = torch.cuda.current_stream()
+    out = {}
+    for name, la, lb in (("NN", 1, 1), ("NT", 1, 0), ("TN", 0, 1), ("TT", 0, 0)):
+        ms, _, span = timed_launches(lambda: rs.gemm(dC, dA, dB, M, N, K, 0, la, lb, stream=stream), steps, warmup)
+        row = summary(M, N, K, ms, span)
+        out[name] = {"avg_tflops": row["avg_tflops"], "min_time_tflops": row["min_time_tflops"],
+                     "pct_peak_avg": row["pct_peak_avg"]}
     return out
 
 
@@ -446,7 +506,10 @@ def main():
     ap.add_argument("--no-layouts", action="store_true", help="skip the per-layout and 8192^3 table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-context", action="store_true", help="skip the vendor-library context")
-    ap.add_argument("--counters", action="store_true", help="also collect rocprofv3 counters")
+    ap.add_argument("--counters", action="store_true",
+                    help="also write the counter summary under profiles/ (the counters themselves are "
+                         "collected by default)")
+    ap.add_argument("--no-counters", action="store_true", help="skip the rocprofv3 counter passes")
     ap.add_argument("--inner", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -476,21 +539,29 @@ def main():
     ms_per_step = wall_ms / args.steps
     cfg = rs.find_config(M, N, K).as_dict()
 
-    counters = None
-    if args.counters:
-        counters = counters_report(args.steps, args.warmup)
-        write_counter_summary(counters, avg_ms)
+    counters, counters_error = None, None
+    if not args.no_counters:
+        try:
+            counters = counters_report(args.steps, args.warmup)
+        except (RuntimeError, OSError, subprocess.SubprocessError) as e:
+            counters_error = f"{type(e).__name__}: {e}"[:200]
+            if args.counters:
+                sys.exit(f"bench.py: --counters asked for, but the rocprofv3 passes failed ({counters_error})")
+    if counters is not None and counters.get("hbm_bytes_per_launch") is not None:
+        if args.counters:
+            write_counter_summary(counters, avg_ms)
         counters.pop("raw", None)
-        traffic = counters.get("hbm_bytes_per_launch")
-        traffic_source = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes of this run"
+        traffic = counters["hbm_bytes_per_launch"]
+        traffic_source = "this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes"
     else:
         traffic = read_traffic()
         traffic_source = (None if traffic is None else
                           "profiles/sgemm_mfma_4096_rrr_counters.txt: rocprofv3 --pmc passes of an "
-                          "earlier `bench.py --counters` run of this workload, not measured in this run")
+                          "earlier `bench.py --counters` run of this workload, not measured in this run"
+                          + (f" ({counters_error})" if counters_error else ""))
 
     line = {
-        "metric": "SGEMM TFLOPS (avg & min) at 4096^3; % of MI355X FP32 MFMA peak",
+        "metric": "SGEMM TFLOPS (avg & min) at 4096^3 NN/NT/TN/TT; % of MI355X FP32 MFMA peak",
         "value": round(tflops(M, N, K, ms_per_step), 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -518,9 +589,14 @@ def main():
     }
     if counters is not None:
         line["counters"] = counters
+        for k in ("mfma_busy_pct", "lds_bank_conflict_pct"):
+            if k in counters:
+                line["roofline"][k] = counters[k]
+    line["dense_4096"] = bench_dense_4096(rs, args.steps, args.warmup)
     if not args.no_layouts:
         line["layouts"] = bench_layouts(rs, (1024, 2048, 4096, 8192), args.steps, args.warmup)
         line["shapes_row_major"] = bench_shapes(rs, args.steps, args.warmup)
+        line["held_out"] = bench_held_out(rs, args.steps, args.warmup)
     if not args.no_context:
         line["context"] = bench_context((4096, 8192), args.steps, args.warmup)
         ceiling = mfma_only_kernel()

@@ -78,8 +78,9 @@ enum
  *                       1 = a second kernel; 2 = the GEMM launch itself, whenever it can (the wave
  *                       that completes a tile's counter adds the tile's parts up: no second
  *                       launch, but one wave reads all parts of its share of the tile);
- *                       0 = the library decides (in the launch for products of at least 8 GFLOP
- *                       whose waves have at most 48 KB to add up, else a second kernel).
+ *                       0 = the library decides, which at present means a second kernel: with
+ *                       the wait for its write-through stores that the scheme needs, the launch
+ *                       lost to the second kernel on every problem it was timed on.
  *                       The result is the same bit for bit either way (same order of addition)
  */
 typedef struct rocm_sgemm_config
@@ -141,6 +142,15 @@ int rocm_sgemm_f32_no_alloc(int          layout_c,
                             size_t       N,
                             size_t       K,
                             void*        stream);
+
+/*
+ * Bytes of workspace rocm_sgemm_f32 would use for the partial products of this problem under the
+ * config it plans (0: the plan neither splits K nor deals out a stream-K tail); what
+ * rocm_sgemm_f32_no_alloc compares with ROCM_SGEMM_NO_ALLOC_SCRATCH_BYTES.  Host only: nothing is
+ * allocated, launched or read.  No counterpart in the reference, which never splits K
+ * (rocm_sgemm/src/gemm.cpp:21-25: one block per output tile).
+ */
+int rocm_sgemm_workspace_bytes(int layout_c, int layout_a, int layout_b, size_t M, size_t N, size_t K, size_t* bytes);
 
 /*
  * Same product with an explicit config instead of the table lookup.  Replaces the tuner's
@@ -232,7 +242,7 @@ int rocm_sgemm_nearest_config(size_t M, size_t N, size_t K, int layout_a, int la
  * CU, reduced when it would exceed four per CU); the cost model below then prices that config,
  * those of the next three nearest entries and the larger direct-to-LDS tile shapes of the family
  * at split_k 1, 2, 3, 4, 6 and 8, and the cheapest replaces the nearest entry's config if it is
- * expected to be at least 4 % faster (distance in log size says nothing about how a tile shape
+ * expected to be at least 6 % faster (distance in log size says nothing about how a tile shape
  * divides M and N or how many tiles are left for 256 CUs).  Host-only, needs no GPU.
  */
 int rocm_sgemm_find_config(size_t M, size_t N, size_t K, int layout_a, int layout_b, int layout_c,

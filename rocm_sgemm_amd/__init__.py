@@ -30,7 +30,8 @@ NO_ALLOC_SCRATCH_BYTES = 128 * 1024 * 1024
 
 # Every extern "C" symbol declared in include/rocm_sgemm.h.
 C_SYMBOLS = (
-    "rocm_sgemm_f32", "rocm_sgemm_f32_no_alloc", "rocm_sgemm_f32_with_config", "rocm_sgemm_f32_strided_batched",
+    "rocm_sgemm_f32", "rocm_sgemm_f32_no_alloc", "rocm_sgemm_workspace_bytes", "rocm_sgemm_f32_with_config",
+    "rocm_sgemm_f32_strided_batched",
     "rocm_sgemm_f32_strided_batched_with_config", "rocm_sgemm_nearest_config", "rocm_sgemm_find_config",
     "rocm_sgemm_find_config_batched", "rocm_sgemm_predict_us",
     "rocm_sgemm_table_size", "rocm_sgemm_table_entry", "rocm_sgemm_family_size",
@@ -109,6 +110,8 @@ def lib():
                                       c_size_t, c_size_t, c_void_p]
     handle.rocm_sgemm_f32_with_config.argtypes = [cfg_p] + handle.rocm_sgemm_f32.argtypes
     handle.rocm_sgemm_f32_no_alloc.argtypes = handle.rocm_sgemm_f32.argtypes
+    handle.rocm_sgemm_workspace_bytes.argtypes = [c_int, c_int, c_int, c_size_t, c_size_t, c_size_t,
+                                                  ctypes.POINTER(c_size_t)]
     c_float, c_ll = ctypes.c_float, ctypes.c_longlong
     handle.rocm_sgemm_f32_strided_batched.argtypes = [
         c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_ll, c_void_p, c_size_t, c_ll, c_float,
@@ -182,6 +185,15 @@ def gemm_no_alloc(C, A, B, M, N, K, layout_c="row_major", layout_a="row_major", 
     STATUS_WORKSPACE_TOO_LARGE."""
     _check(lib().rocm_sgemm_f32_no_alloc(_layout(layout_c), _layout(layout_a), _layout(layout_b),
                                          _ptr(C), _ptr(A), _ptr(B), M, N, K, _stream(stream)))
+
+
+def workspace_bytes(M, N, K, layout_a="row_major", layout_b="row_major", layout_c="row_major"):
+    """Bytes of workspace `gemm` would use for the partial products of this problem under the config
+    it plans (0 = none); what `gemm_no_alloc` holds against NO_ALLOC_SCRATCH_BYTES.  Host only."""
+    out = ctypes.c_size_t()
+    _check(lib().rocm_sgemm_workspace_bytes(_layout(layout_c), _layout(layout_a), _layout(layout_b), M, N, K,
+                                            ctypes.byref(out)))
+    return out.value
 
 
 def gemm_with_config(config, C, A, B, M, N, K, layout_c="row_major", layout_a="row_major",

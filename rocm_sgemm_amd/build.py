@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Builds librocm_sgemm.so (gfx950), the tuner trial binary, bench_float and kernel_phases with hipcc, in-tree.
+"""Builds librocm_sgemm.so (gfx950), the tuner trial binary, bench_float, kernel_phases and issue_cost with hipcc, in-tree.
 
 Plays the role of the reference's CMake targets `rocm_sgemm` and `tuner`
 (reference rocm_sgemm/CMakeLists.txt:11-89): run the config generator, compile one translation
@@ -29,6 +29,8 @@ BENCH_SRC = os.path.join(PKG_DIR, "benchmark", "bench_float.cpp")
 BENCH_PATH = os.path.join(PKG_DIR, "benchmark", "bench_float")
 PHASES_SRC = os.path.join(PKG_DIR, "benchmark", "kernel_phases.hip")
 PHASES_PATH = os.path.join(PKG_DIR, "benchmark", "kernel_phases")
+ISSUE_SRC = os.path.join(PKG_DIR, "benchmark", "issue_cost.hip")
+ISSUE_PATH = os.path.join(PKG_DIR, "benchmark", "issue_cost")
 CALLER_SRC = os.path.join(REPO_DIR, "tests", "cxx", "reference_style_caller.cpp")
 CALLER_PATH = os.path.join(REPO_DIR, "tests", "cxx", "reference_style_caller")
 # a caller that includes the reference's own host headers by path: built only where that tree is
@@ -232,6 +234,13 @@ def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR, side
             raise RuntimeError("kernel_phases failed to build:\n" + (proc.stdout + proc.stderr)[-4000:])
         if verbose:
             print(f"linked {PHASES_PATH}")
+        # what an instruction costs next to back-to-back MFMAs: a microbenchmark, links nothing of the library
+        cmd = [hipcc()] + COMMON_FLAGS + ["-x", "hip", ISSUE_SRC, "-o", ISSUE_PATH]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError("issue_cost failed to build:\n" + (proc.stdout + proc.stderr)[-4000:])
+        if verbose:
+            print(f"linked {ISSUE_PATH}")
     return LIB_PATH
 
 

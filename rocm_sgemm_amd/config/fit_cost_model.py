@@ -33,23 +33,23 @@ CUS = 256
 
 # name: (value compiled into csrc/planner.cpp, lower bound, upper bound)
 CONSTANTS = {
-    "eff_128x64": (1.0, 0.5, 1.0),   # sustained matrix-pipe efficiency by wave-tile area >= 8192
-    "eff_64x64": (0.953, 0.5, 1.0),    # >= 4096
-    "eff_64x32": (0.97, 0.4, 1.0),    # >= 2048
-    "eff_32x32": (0.921, 0.3, 1.0),    # smaller
-    "k_tile_64": (0.951, 0.9, 1.3),
-    "mfma_16": (0.947, 0.8, 1.1),
-    "register_staged": (0.911, 0.7, 1.1),
-    "stages_3_4": (0.955, 0.9, 1.1),
-    "masked_4_byte": (0.892, 0.6, 1.1),   # problem not all multiples of 4
-    "masked_16_byte": (0.922, 0.8, 1.05),  # ragged multiples of 4
-    "l2_tbs": (18.75, 3.0, 40.0),           # L2 -> LDS panel bandwidth over the chip
-    "l2_tbs_4_byte": (11.64, 2.0, 40.0),
-    "launch_us": (5.86, 2.0, 15.0),
-    "split_us": (2.82, 0.0, 15.0),
-    "split_tbs": (3.68, 1.0, 10.0),
-    "tail_us": (5.72, 0.0, 20.0),
-    "tail_tbs": (5.57, 1.0, 12.0),
+    "eff_128x64": (0.992, 0.5, 1.0),   # sustained matrix-pipe efficiency by wave-tile area >= 8192
+    "eff_64x64": (0.989, 0.5, 1.0),    # >= 4096
+    "eff_64x32": (1.0, 0.4, 1.0),    # >= 2048
+    "eff_32x32": (0.978, 0.3, 1.0),    # smaller
+    "k_tile_64": (0.953, 0.9, 1.3),
+    "mfma_16": (0.931, 0.8, 1.1),
+    "register_staged": (1.036, 0.7, 1.1),
+    "stages_3_4": (0.957, 0.9, 1.1),
+    "masked_4_byte": (0.872, 0.6, 1.1),   # problem not all multiples of 4
+    "masked_16_byte": (0.932, 0.8, 1.05),  # ragged multiples of 4
+    "l2_tbs": (40.0, 3.0, 40.0),           # L2 -> LDS panel bandwidth over the chip
+    "l2_tbs_4_byte": (11.31, 2.0, 40.0),
+    "launch_us": (5.75, 2.0, 15.0),
+    "split_us": (2.45, 0.0, 15.0),
+    "split_tbs": (3.46, 1.0, 10.0),
+    "tail_us": (5.57, 0.0, 20.0),
+    "tail_tbs": (4.77, 1.0, 12.0),
 }
 NAMES = list(CONSTANTS)
 

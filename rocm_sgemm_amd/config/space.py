@@ -18,7 +18,7 @@ describe a wave32 VALU kernel (thread tiles, threads_n); an MFMA kernel is descr
                         through LDS (1 = none); block size = 64 * waves_m * waves_n * waves_k
     split_k, group_m    launch-time only: K slices and tile-order band height
     partial_sums        launch-time only: who adds up the partial tiles of a K split or a stream-K
-                        tail: 0 = the library decides, 1 = a second kernel, 2 = the GEMM launch
+                        tail: 0 = the library decides (a second kernel), 1 = a second kernel, 2 = the GEMM launch
     wave_slots          launch-time only: 0 = deal the K range of a short last wave of tiles out
                         to all CUs (stream-K tail; slots asked from the runtime), 1 = never
 
@@ -33,8 +33,8 @@ NUM_CU = 256
 NUM_XCD = 8
 
 PARAM_SPACE = {
-    "macro_m": [32, 64, 128, 256],
-    "macro_n": [32, 64, 128, 256],
+    "macro_m": [16, 32, 64, 128, 256],
+    "macro_n": [16, 32, 64, 128, 256],
     "k_tile": [16, 32, 64, 128],
     "waves_m": [1, 2, 4],
     "waves_n": [1, 2, 4],
@@ -169,6 +169,12 @@ _BASE_SHAPES = [
     (64, 32, 64, 1, 1, 32, 3, 4),
     (128, 64, 32, 2, 1, 32, 3, 2),
     (64, 64, 128, 1, 1, 32, 2, 4),
+    # 16-row tiles on v_mfma_f32_16x16x4_f32 for problems with M or N <= 16: half the wasted rows of
+    # a 32-row tile, and stages small enough for two or three workgroups per CU, i.e. more loads in
+    # flight for what is a stream over the other operand (found by the tuner's exploration mode:
+    # 4096 x 16 x 4096 14.8 against 16.9 us, 16 x 16384 x 1024 13.2 against 13.9)
+    (16, 32, 64, 1, 1, 16, 4, 2),
+    (16, 64, 64, 1, 1, 16, 3, 2),
     # register-staged (stages = 0): K-tiles of 16 for very shallow problems
     (256, 128, 16, 2, 2, 32, 0, 1),
 ]

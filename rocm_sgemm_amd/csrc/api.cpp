@@ -2,6 +2,7 @@
 // (include/rocm_sgemm/gemm.hpp; reference rocm_sgemm/src/gemm.cpp:8-111).
 
 #include <stdexcept>
+#include <cstdint>
 #include <string>
 
 #include <rocm_sgemm.h>
@@ -69,6 +70,23 @@ int rocm_sgemm_f32_no_alloc(int          layout_c,
     problem.no_alloc = true;
     std::string error;
     const int   status = run_gemm(config, problem, static_cast<hipStream_t>(stream), error);
+    return status == ROCM_SGEMM_STATUS_OK ? status : fail(status, error);
+}
+
+int rocm_sgemm_workspace_bytes(int layout_c, int layout_a, int layout_b, size_t M, size_t N, size_t K, size_t* bytes)
+{
+    using namespace rocm_sgemm::detail;
+    if(bytes == nullptr || M == 0 || N == 0 || K == 0)
+    {
+        return fail(ROCM_SGEMM_STATUS_INVALID_ARG, "matrix dimensions must be positive and `bytes` non-null");
+    }
+    const rocm_sgemm_config config = plan_config(M, N, K, layout_a, layout_b, layout_c);
+    // the size does not depend on the operands' addresses; these are never dereferenced
+    float* const nowhere = reinterpret_cast<float*>(static_cast<uintptr_t>(256));
+    gemm_problem problem{layout_c, layout_a, layout_b, nowhere, nowhere, nowhere, M, N, K, 0, 0, 0, 0, 0, 0, 1, 1.0f, 0.0f};
+    problem.workspace_bytes_out = bytes;
+    std::string error;
+    const int   status = run_gemm(config, problem, nullptr, error);
     return status == ROCM_SGEMM_STATUS_OK ? status : fail(status, error);
 }
 
@@ -296,6 +314,12 @@ const char* rocm_sgemm_version(void)
 namespace rocm_sgemm
 {
 
+namespace detail
+{
+// Never runs: gemm<>() launches it over an empty grid to leave a HIP error for a refused call.
+__global__ void refused_call_marker() {}
+} // namespace detail
+
 template<m_layout layout_C, m_layout layout_A, m_layout layout_B, class T>
 __host__ void gemm(T* C, T* A, T* B, size_t M, size_t N, size_t K, hipStream_t& stream)
 {
@@ -313,11 +337,20 @@ __host__ void gemm(T* C, T* A, T* B, size_t M, size_t N, size_t K, hipStream_t& 
     // caller's hipPeekAtLastError (kernel_launcher.hpp:96-98, test/gemm/test.cpp:69); its one
     // exception is the missing kernel (kernel_launcher.hpp:89-94).  Same here, so that a caller
     // written without a try block is never terminated: a refused call (zero dimension, null
-    // pointer, dimension above 2^31 - 4097) enqueues nothing and leaves its reason in
-    // rocm_sgemm_last_error().
+    // pointer, dimension above 2^31 - 4097) enqueues nothing, leaves its reason in
+    // rocm_sgemm_last_error() - and leaves a HIP error behind, as the reference's launch of an
+    // empty grid does, so that the check its callers already make after every call
+    // (hipPeekAtLastError, CHECK_LAST_HIP_ERROR) sees the failure instead of silently finding the
+    // old contents of C.
     if(status == ROCM_SGEMM_STATUS_NO_KERNEL)
     {
         throw std::runtime_error(rocm_sgemm_last_error());
+    }
+    if(status == ROCM_SGEMM_STATUS_INVALID_ARG)
+    {
+        // a launch over an empty grid: rejected by the runtime (hipErrorInvalidConfiguration),
+        // nothing is enqueued
+        hipLaunchKernelGGL(detail::refused_call_marker, dim3(0), dim3(1), 0, stream);
     }
 }
 

@@ -463,7 +463,9 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     // An operand can travel 16 bytes per lane when every line of it starts on a 16-byte boundary
     // (a misaligned load of that size faults) and, if it is stored depth-contiguous, its rows end
     // on one (whole 16-byte pieces beyond K are dropped; one straddling the end of a row could
-    // not be).  Otherwise it travels 4 bytes per lane, which needs no alignment.
+    // not be).  Only two masked kernels exist per shape: both operands 16 bytes per lane, or both
+    // 4 bytes per lane (which needs no alignment), so one operand that cannot go wide takes the
+    // other with it.
     const bool x_aligned = aligned16(args.X) && args.ldx % 4 == 0 && (p.batch == 1 || args.stride_x % 4 == 0);
     const bool y_aligned = aligned16(args.Y) && args.ldy % 4 == 0 && (p.batch == 1 || args.stride_y % 4 == 0);
     const bool out_aligned   = to_workspace
@@ -474,10 +476,9 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     // Full tiles of 16-byte aligned lines: the kernel without masks.  Anything else runs an
     // edge-masked kernel: a direct-to-LDS shape the one with 16-byte loads if both operands allow
     // them, else the one with 4-byte loads; a register-staged shape its own.
-    const bool      x_wide   = x_aligned && (!x_kc || args.depth % 4 == 0);
-    const bool      y_wide   = y_aligned && (!y_kc || args.depth % 4 == 0);
-    const launch_fn masked   = row->launch[x_kc ? 1 : 0][y_kc ? 1 : 0][2];
-    const int       variant  = full ? 0 : (masked == nullptr ? 1 : (x_wide && y_wide ? 2 : 3));
+    const bool      both_wide = x_aligned && y_aligned && ((!x_kc && !y_kc) || args.depth % 4 == 0);
+    const launch_fn masked    = row->launch[x_kc ? 1 : 0][y_kc ? 1 : 0][2];
+    const int       variant   = full ? 0 : (masked == nullptr ? 1 : (both_wide ? 2 : 3));
     launch_fn       fn       = row->launch[x_kc ? 1 : 0][y_kc ? 1 : 0][variant];
 
     // Stream-K tail.  The matrix pipes of the GPU are saturated by W workgroups (one per CU for
@@ -533,29 +534,31 @@ int run_gemm(const rocm_sgemm_config& c, const gemm_problem& p, hipStream_t stre
     {
         workspace_floats = static_cast<size_t>(args.tail_groups) * 2 * bm * bn;
     }
-    // Who adds the partial tiles up: the launch itself (the wave that completes a tile's counter,
-    // see kernel::gemm_args::counters) or a second kernel.  The first saves a launch and the
-    // write-back of the partial tiles at the end of the GEMM kernel, and the summing of one tile
-    // overlaps with the multiplication of others: 2 to 10 % on products of 80 us and more.  But
-    // every wave waits for its stores and its ticket, and the wave that adds up reads all parts of
-    // its share one after the other: on products of 20 to 45 us, where all tiles finish together
-    // and nothing overlaps, it costs 2 to 5 us more than the second launch.  And one wave reads at
-    // a few GB/s, so its share must be little data.  Hence, unless the config says otherwise:
-    // in the launch for products of at least 8 GFLOP whose waves have at most 48 KB to add up.
+    // Who adds the partial tiles up: a second kernel, or - only where the config asks for it
+    // (partial_sums = 2) - the launch itself: the wave that completes a tile's counter, see
+    // kernel::gemm_args::counters.  The second saves a launch and the summing of one tile overlaps
+    // with the multiplication of others, but every wave must wait until its write-through stores
+    // have been acknowledged before it may draw its ticket, and the wave that adds up reads all
+    // parts of its share one after the other.  Measured after that wait went in (it is what makes
+    // the scheme correct) and the main loop lost its stalls: the second kernel wins everywhere it
+    // was tried - 2560^3 237.5 against 255.1 us, 1024 x 1024 x 16384 (64 x 64 x 64, four waves
+    // along K, split 2) 238.4 against 245.0, 1024 x 1024 x 4096 69.5 against 78.1, 768 x 384 x 2304
+    // 24.5 against 27.3 - so it is the default (partial_sums = 0 and 1 mean the same); the tuner
+    // still times both and records a 2 where the launch wins.
     // (Possible at all only with at most four waves that own at most a 64 x 64 share of the tile
     // each, kernel::tile_config::SUMS_IN_LAUNCH, 32-bit byte offsets into a partial matrix, and
     // counters for every (batch, tile, wave).)
     const int    waves_per_group = wm * wn * (c.waves_k > 1 ? c.waves_k : 1);
     const size_t counters_needed
         = static_cast<size_t>(p.batch) * static_cast<size_t>(args.tail_groups > 0 ? tail_tiles : tiles) * waves_per_group;
-    const long long parts          = args.tail_groups > 0 ? (k_tiles + args.tail_per - 1) / args.tail_per + 1 : split;
-    const long long bytes_per_wave = parts * bm * bn * 4ll / waves_per_group;
-    const double    flop           = 2.0 * static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K)
-                        * static_cast<double>(p.batch);
-    const bool      possible = !scaled && (split > 1 || args.tail_groups > 0) && counters_needed <= counter_slots
+    const bool possible = !scaled && (split > 1 || args.tail_groups > 0) && counters_needed <= counter_slots
                           && bm * bn / waves_per_group <= 64 * 64 && waves_per_group <= 4 && count < (1ull << 29);
-    bool in_launch = possible
-                     && (c.partial_sums == 2 || (c.partial_sums == 0 && flop >= 8.0e9 && bytes_per_wave <= 48 * 1024));
+    bool       in_launch = possible && c.partial_sums == 2;
+    if(p.workspace_bytes_out != nullptr)
+    {
+        *p.workspace_bytes_out = workspace_floats * sizeof(float);
+        return ROCM_SGEMM_STATUS_OK;
+    }
     void* workspace_base = nullptr;
     if(workspace_floats > 0 && p.no_alloc)
     {

@@ -39,7 +39,7 @@ const rocm_sgemm_config& select_config(const tuned_entry*       table,
 /// table entry gets its entry; anything else the cheapest, by the cost model below, of the
 /// nearest entry's config (K split fitted to the problem's own tile count), those of the next
 /// three nearest entries and the larger direct-to-LDS shapes of the family at split_k 1, 2, 3, 4, 6, 8 -
-/// the nearest entry's config stays unless another is predicted at least 4 % faster.
+/// the nearest entry's config stays unless another is predicted at least 6 % faster.
 rocm_sgemm_config plan_config(size_t m, size_t n, size_t k, int layout_a, int layout_b, int layout_c,
                               size_t batch = 1);
 
@@ -77,6 +77,9 @@ struct gemm_problem
     /// Partial products go to the fixed scratch array of the GPU instead of an allocated workspace;
     /// a problem that needs more than the array holds is refused.
     bool no_alloc = false;
+    /// Query only: when set, run_gemm stores the bytes of workspace the call would need for its
+    /// partial products there (0 = none) and returns before any allocation or launch.
+    size_t* workspace_bytes_out = nullptr;
 };
 
 /// Validates, resolves the kernel and enqueues it.  Returns a ROCM_SGEMM_STATUS_* value and, on

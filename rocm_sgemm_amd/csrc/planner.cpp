@@ -196,47 +196,50 @@ bool tail_applies(const rocm_sgemm_config& c, long long tiles, long long k_tiles
 // or the K split add their second pass; every launch a fixed cost.  The constants are a
 // least-squares fit (log time, weighted towards each problem's fastest configs) to tuner sweeps of
 // the whole family over 79 problems between 192 x 192 x 8192 and 7052 x 2436 x 856, regular and
-// ragged, on MI355X; choosing each problem's config by this model lands within 4.7 % of its fastest
-// on average (4.2 - 6.5 % on held-out thirds).  Used to choose among candidate configs for problems that are not table entries, so
+// ragged, on MI355X (6 424 timed configs); choosing each problem's config by this model lands
+// within 4.5 % of its fastest on average (3.7 - 6.3 % on held-out thirds, worst case 30 %).  Since
+// the main loop lost its stalls the efficiencies of all wave-tile sizes are within 2 % of each
+// other.  Used to choose among candidate configs for problems that are not table entries, so
 // mainly the ordering matters.
 double predict_us(const rocm_sgemm_config& c, size_t m, size_t n, size_t k, size_t batch)
 {
     const int    waves     = c.waves_m * c.waves_n * (c.waves_k > 1 ? c.waves_k : 1);
     const int    per_cu    = waves >= 4 ? 1 : 4 / (waves < 1 ? 1 : waves);
     const double wave_area = static_cast<double>(c.macro_m / c.waves_m) * (c.macro_n / c.waves_n);
-    double       eff = wave_area >= 8192 ? 1.000 : wave_area >= 4096 ? 0.953 : wave_area >= 2048 ? 0.970 : 0.921;
-    if(c.k_tile >= 64) eff *= 0.951;
-    if(c.mfma == 16) eff *= 0.947;
-    if(c.stages == 0) eff *= 0.911;
-    if(c.stages >= 3) eff *= 0.955;
+    double       eff = wave_area >= 8192 ? 0.992 : wave_area >= 4096 ? 0.989 : wave_area >= 2048 ? 1.000 : 0.978;
+    if(c.k_tile >= 64) eff *= 0.953;
+    if(c.mfma == 16) eff *= 0.931;
+    if(c.stages == 0) eff *= 1.036;
+    if(c.stages >= 3) eff *= 0.957;
     // ragged problems run the masked kernels: 16-byte loads when every dimension is a multiple
     // of 4, 4-byte loads otherwise
     const bool aligned = m % 4 == 0 && n % 4 == 0 && k % 4 == 0;
     const bool full    = m % c.macro_m == 0 && n % c.macro_n == 0 && k % c.k_tile == 0;
     if(!aligned)
-        eff *= 0.892;
+        eff *= 0.872;
     else if(!full)
-        eff *= 0.922;
+        eff *= 0.932;
     // the products of a batch are one launch: their tiles fill the waves together
     const long long tiles   = static_cast<long long>((m + c.macro_m - 1) / c.macro_m) * ((n + c.macro_n - 1) / c.macro_n)
                               * static_cast<long long>(batch);
     const long long k_tiles = static_cast<long long>((k + c.k_tile - 1) / c.k_tile);
     const double    kd      = static_cast<double>(k);
     const double    compute = 2.0 * c.macro_m * c.macro_n * kd / (614.5e3 * eff); // one CU's matrix pipes
-    // L2 -> LDS: 18.75 TB/s over the CUs; 11.64 TB/s for the 4-byte loads of a direct-to-LDS shape,
+    // L2 -> LDS: 40 TB/s over the CUs (the fit's upper bound: with 16-byte loads this term no longer
+    // binds any shape of the family); 11.31 TB/s for the 4-byte loads of a direct-to-LDS shape,
     // which are bound by the number of load instructions
-    const double    l2_tbs  = !aligned && c.stages != 0 ? 11.64 : 18.75;
+    const double    l2_tbs  = !aligned && c.stages != 0 ? 11.31 : 40.0;
     const double    panels  = (c.macro_m + c.macro_n) * kd * 4.0 / (l2_tbs * 1.0e6 / model_cus);
     const double    tile_us = std::sqrt(std::sqrt(compute * compute * compute * compute + panels * panels * panels * panels)) * per_cu;
     const double    out_mb  = static_cast<double>(m) * n * 4.0 / 1.0e6 * static_cast<double>(batch);
-    double          t       = 5.86; // launch, first loads, last stores
+    double          t       = 5.75; // launch, first loads, last stores
     if(c.split_k > 1)
     {
         const long long split  = c.split_k < k_tiles ? c.split_k : k_tiles;
         const long long groups = tiles * split;
         const long long slots  = model_cus * per_cu;
         t += static_cast<double>((groups + slots - 1) / slots) * tile_us / split;
-        t += 2.82 + (split + 1) * out_mb / 3.68; // second pass: launch gap, partials at ~3.7 TB/s
+        t += 2.45 + (split + 1) * out_mb / 3.46; // second pass: launch gap, partials at ~3.5 TB/s
         return t;
     }
     long long slots = 0, r = 0;
@@ -247,8 +250,8 @@ double predict_us(const rocm_sgemm_config& c, size_t m, size_t n, size_t k, size
         if(tail)
         {
             const double tile_mb = c.macro_m * c.macro_n * 4.0 / 1.0e6;
-            // second pass: launch gap, the segments at ~5.6 TB/s
-            t += tile_us * static_cast<double>(r) / slots + 5.72 + (2.0 * slots + r) * tile_mb / 5.57;
+            // second pass: launch gap, the segments at ~4.8 TB/s
+            t += tile_us * static_cast<double>(r) / slots + 5.57 + (2.0 * slots + r) * tile_mb / 4.77;
         }
         else
         {
@@ -315,9 +318,10 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     // problem's M and N and to how many tiles that leaves for 256 CUs.  So the cost model also
     // prices the configs of the four nearest entries of the same layouts and kind, and every
     // direct-to-LDS tile shape of the family with 32 x 32 MFMAs and tiles of at least 64 x 64 (or
-    // smaller ones with waves along K, which keep a large wave tile) at
+    // smaller ones with waves along K, which keep a large wave tile; the 16-row tiles of 16 x 16
+    // MFMAs where the problem has at most 16 rows or columns) at
     // split_k 1, 2, 3, 4, 6 and 8; the cheapest of them replaces the nearest entry's config only if
-    // the model expects it to be at least 4 % faster (about the model's own error).
+    // the model expects it to be at least 6 % faster (the model's own error on held-out problems).
     const auto aligned_kind = [](size_t a, size_t b, size_t c) { return a % 4 == 0 && b % 4 == 0 && c % 4 == 0; };
     constexpr int   max_candidates = 4;
     const log_size  here  = logs_of(m, n, k);
@@ -353,7 +357,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     const double nearest_us = best_us;
     const auto   consider   = [&](const rocm_sgemm_config& c) {
         const double us = predict_us(c, m, n, k, batch);
-        if(us < best_us && us <= 0.96 * nearest_us)
+        if(us < best_us && us <= 0.94 * nearest_us)
         {
             best    = c;
             best_us = us;
@@ -369,7 +373,9 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     {
         rocm_sgemm_config s{};
         family_entry(i, &s);
-        if(s.stages < 2 || s.mfma != 32 || ((s.macro_m < 64 || s.macro_n < 64) && s.waves_k <= 1)) continue;
+        if(s.stages < 2 || ((s.macro_m < 64 || s.macro_n < 64) && s.waves_k <= 1)) continue;
+        // 16-row (16-column) tiles of 16 x 16 MFMAs: only where the problem has no more rows (columns)
+        if(s.mfma != 32 && !((s.macro_m == 16 && m <= 16) || (s.macro_n == 16 && n <= 16))) continue;
         const long long k_tiles = static_cast<long long>((k + s.k_tile - 1) / s.k_tile);
         for(const int split : {1, 2, 3, 4, 6, 8})
         {

@@ -27,9 +27,9 @@
 //     as the rows of a depth-contiguous operand end on a 16-byte boundary (K a multiple of 4).
 //     With DGX == 1 (DGY == 1) the same kernel moves X (Y) 4 bytes per lane (buffer_load_dword
 //     ... lds) into the same LDS image, which lifts every alignment requirement on that operand:
-//     odd leading dimension, unaligned pointer, any K.  The granularity is chosen per operand: in
-//     a row-major 1000 x 3000 x 777 product only A's lines (777 floats) are misaligned, B's (3000
-//     floats) still travel 16 bytes per lane.
+//     odd leading dimension, unaligned pointer, any K.  The granularity is a template parameter
+//     per operand, but only the 16 / 16 and the 4 / 4 kernels are compiled: one misaligned operand
+//     moves both to 4-byte loads (a 16 / 4 kernel measured 1 % faster where it applies).
 //   register-staged (NS == 0; the alternative for shapes without an LDS ring):
 //     HBM --128-bit buffer loads--> registers (one K-tile ahead)
 //         --128-bit ds_write, same orientation as in memory--> LDS (two stages)
@@ -222,17 +222,6 @@ struct tile_config
     static_assert(NS == 0 || (NS >= 2 && NS <= 8), "0 (register-staged) or 2..8 LDS stages");
     static_assert(!DTL || (MI / RPL) % CPR == 0, "swizzle must not depend on the MFMA tile index");
 };
-
-// Tunables of the slot schedule (overridable at compile time for experiments).
-#ifndef RSG_READ_SPAN_PCT
-#define RSG_READ_SPAN_PCT 100 // fragment reads of a k-block are spread over this share of its slots
-#endif
-#ifndef RSG_BARRIER_SLOT
-#define RSG_BARRIER_SLOT 0 // slot of the last k-block that carries the barrier
-#endif
-#ifndef RSG_MOVE_SPREAD
-#define RSG_MOVE_SPREAD 0 // 1: spread LDS stores / global loads over all k-blocks but the last
-#endif
 
 namespace impl
 {
@@ -917,13 +906,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
     // Slot assignment.  Reads of a k-block are spread over READ_SPAN slots starting at slot 0 (at
     // the barrier slot in the last k-block); the movement items of the K-tile are spread over
     // the MOVE_KBS first k-blocks.
-    constexpr int BARRIER_SLOT = RSG_BARRIER_SLOT < SLOTS ? RSG_BARRIER_SLOT : SLOTS - 1;
+    constexpr int BARRIER_SLOT = 0; // slot of the last k-block that carries the barrier
     // Single-float loads are four times as many.  A ring of three or more stages has a whole
     // K-tile of slack, so they are spread over all k-blocks but the last; with two stages a load
     // must land before this iteration's barrier, so they are issued as early as two per slot allow.
     constexpr int DENSE_KBS    = impl::max_int(1, (NMOVE + 2 * SLOTS - 1) / (2 * SLOTS));
-    constexpr int MOVE_KBS     = RSG_MOVE_SPREAD ? NKB - 1
-                                 : (DTL && (DGX == 1 || DGY == 1)) ? (NS >= 3 || DENSE_KBS > NKB - 1 ? NKB - 1 : DENSE_KBS)
+    constexpr int MOVE_KBS     = (DTL && (DGX == 1 || DGY == 1)) ? (NS >= 3 || DENSE_KBS > NKB - 1 ? NKB - 1 : DENSE_KBS)
                                                     : 1;
     constexpr int MOVE_SLOTS   = MOVE_KBS * SLOTS;
     // One K-tile of the pipeline: K-tile t sits in stage `cur_c`.  With `ragged_c` false the caller
@@ -941,7 +929,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MIN_WAVES_PER_SIMD) void sgemm_mfma_k
             constexpr bool last_kb  = kb == NKB - 1;
             constexpr int  read_off = last_kb ? BARRIER_SLOT : 0;
             constexpr int  read_span
-                = impl::max_int(1, (SLOTS - read_off) * RSG_READ_SPAN_PCT / 100);
+                = impl::max_int(1, SLOTS - read_off); // reads spread over the rest of the k-block
             impl::static_for<0, SLOTS>([&](auto m_c) {
                 constexpr int m = decltype(m_c)::value;
                 constexpr int r = m / (TM * TN);

@@ -298,6 +298,38 @@ def test_cxx_template_symbols_match_c_abi(la, lb, lc):
     assert np.array_equal(dC.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+def test_refused_cxx_call_leaves_a_hip_error_and_c_untouched():
+    """A zero dimension or a null pointer: the C++ entry point throws nothing and enqueues nothing,
+    but the check the reference's callers make after every call (hipPeekAtLastError,
+    reference test/gemm/test.cpp:69) must see a failure, as it does after the reference's launch of
+    an empty grid."""
+    import torch
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipPeekAtLastError.restype = ctypes.c_int
+    hip.hipGetLastError.restype = ctypes.c_int
+    fn = getattr(rs.lib(), rs.cxx_symbol(0, 0, 0))
+    fn.restype = None
+    fn.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_size_t] * 3 + [ctypes.POINTER(ctypes.c_void_p)]
+    dA = torch.ones(64 * 64, dtype=torch.float32, device="cuda:0")
+    dC = torch.full((64 * 64,), 7.0, dtype=torch.float32, device="cuda:0")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    hip.hipGetLastError()  # start clean
+    for args in ((dC.data_ptr(), dA.data_ptr(), dA.data_ptr(), 0, 64, 64),
+                 (dC.data_ptr(), None, dA.data_ptr(), 64, 64, 64)):
+        _announce("refused_cxx_call", args[3:])
+        fn(*args, ctypes.byref(stream))
+        assert hip.hipPeekAtLastError() != 0
+        assert hip.hipGetLastError() != 0 and hip.hipPeekAtLastError() == 0  # reading it clears it
+        assert "must be" in rs.lib().rocm_sgemm_last_error().decode()
+    torch.cuda.synchronize()
+    assert bool((dC == 7.0).all())
+    # and a good call after it works and leaves no error
+    fn(dC.data_ptr(), dA.data_ptr(), dA.data_ptr(), 64, 64, 64, ctypes.byref(stream))
+    torch.cuda.synchronize()
+    assert hip.hipPeekAtLastError() == 0 and bool((dC == 64.0).all())
+
+
 def test_runs_on_a_side_stream_without_blocking_semantics():
     import torch
     M, N, K = 256, 256, 256
@@ -425,6 +457,32 @@ def test_kernel_phases_accounts_for_a_launch():
         assert busy is not None and 50.0 <= float(busy.group(1)) <= 100.5, block
         each = re.search(r"back to back: ([\d.]+) us each = ([\d.]+) TFLOP/s", block)
         assert each is not None and 40.0 < float(each.group(2)) < 157.3, block
+
+
+def test_issue_cost_of_instructions_next_to_mfmas():
+    """issue_cost measures what one instruction of each kind adds to a stream of back-to-back
+    MFMAs.  The design of the main loop rests on two of its findings: a vector-ALU instruction
+    costs several cycles of matrix-pipe time (about 13 measured), scalar instructions, LDS reads,
+    direct-to-LDS loads and barriers next to nothing."""
+    import os
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rocm_sgemm_amd",
+                       "benchmark", "issue_cost")
+    _announce("issue_cost", exe)
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    alone = float(re.search(r"MFMAs alone: ([\d.]+) cycles each", out.stdout).group(1))
+    assert 63.9 <= alone <= 64.6, out.stdout  # a v_mfma_f32_32x32x2_f32 holds the pipe for 64 cycles
+    cost = {(m.group(1).strip(), int(m.group(2))): float(m.group(3))
+            for m in re.finditer(r"^cost (.+?)\s+every\s+(\d+) MFMAs:\s+(-?[\d.]+) cycles", out.stdout, re.M)}
+    assert len(cost) == 9, out.stdout
+    assert 6.0 <= cost[("vector-ALU add", 8)] <= 25.0 and 6.0 <= cost[("vector-ALU add", 1)] <= 25.0, out.stdout
+    assert cost[("two vector-ALU adds", 8)] >= cost[("vector-ALU add", 8)], out.stdout
+    for free in (("four scalar-ALU adds", 1), ("ds_read_b128", 8), ("ds_read_b128", 2),
+                 ("direct-to-LDS load, 16 bytes per lane", 4), ("s_barrier", 16)):
+        assert cost[free] <= 2.0, (free, out.stdout)
+    assert cost[("direct-to-LDS load, 4 bytes per lane", 1)] <= 3.0, out.stdout
 
 
 def test_bench_float_l2_to_lds_probe():
