@@ -218,20 +218,20 @@ int main(int argc, char** argv)
             rc |= run_case<tile_config<256, 256, 32, 2, 2, 32, true, false, false, 2, 4, 4, 1>>(
                 "256x256x32, 2x2 waves, 2 stages", 8192, 8192, 8192, 4, 1);
         else if(c == "2048")
-            rc |= run_case<tile_config<128, 128, 32, 2, 2, 32, true, false, false, 2, 4, 4, 1>>(
-                "128x128x32, 2x2 waves, 2 stages", 2048, 2048, 2048, 4, 1);
+            rc |= run_case<tile_config<128, 128, 64, 4, 2, 32, true, false, false, 2, 4, 4, 1>>(
+                "128x128x64, 4x2 waves, 2 stages", 2048, 2048, 2048, 4, 1);
         else if(c == "1024")
-            rc |= run_case<tile_config<64, 32, 64, 1, 1, 32, true, false, false, 3, 4, 4, 4>>(
-                "64x32x64, 4 waves along K, 3 stages", 1024, 1024, 1024, 4, 1);
+            rc |= run_case<tile_config<64, 64, 32, 2, 2, 32, true, false, false, 2, 4, 4, 1>>(
+                "64x64x32, 2x2 waves, 2 stages", 1024, 1024, 1024, 4, 1);
         else if(c == "skinny")
-            rc |= run_case<tile_config<32, 64, 64, 1, 1, 32, true, false, false, 3, 4, 4, 4>>(
-                "32x64x64, 4 waves along K, 3 stages", 128, 4096, 4096, 4, 1);
+            rc |= run_case<tile_config<64, 32, 64, 1, 1, 32, true, false, false, 3, 4, 4, 4>>(
+                "64x32x64, 4 waves along K, 3 stages", 128, 4096, 4096, 4, 1);
         else if(c == "ragged")
             rc |= run_case<tile_config<64, 64, 32, 2, 2, 32, true, false, true, 2, 1, 1, 1>>(
                 "64x64x32, 2x2 waves, 2 stages, masked with 4-byte loads", 1000, 3000, 777, 16, 1);
         else if(c == "deepk")
-            rc |= run_case<tile_config<128, 128, 32, 2, 2, 32, true, false, false, 2, 4, 4, 1>>(
-                "128x128x32, 2x2 waves, 2 stages, K split 8", 1024, 1024, 16384, 2, 8);
+            rc |= run_case<tile_config<64, 64, 128, 1, 1, 32, true, false, false, 2, 4, 4, 4>>(
+                "64x64x128, 4 waves along K, 2 stages", 1024, 1024, 16384, 4, 1);
         else
         {
             std::fprintf(stderr, "unknown case %s (4096 8192 2048 1024 skinny ragged deepk)\n", c.c_str());

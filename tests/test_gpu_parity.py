@@ -445,7 +445,7 @@ def test_kernel_phases_accounts_for_a_launch():
     assert out.returncode == 0, out.stdout + out.stderr
     blocks = out.stdout.strip().split("\n\n")
     assert len(blocks) == 2, out.stdout
-    for block, groups in zip(blocks, (256, 512)):
+    for block, groups in zip(blocks, (256, 256)):
         rows = re.findall(r"^\s+(\d)\s+(\d+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s+(\d+) MHz",
                           block, re.M)
         assert len(rows) == 8 and sum(int(r[1]) for r in rows) == groups, block
