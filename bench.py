@@ -419,6 +419,11 @@ def counters_report(steps, warmup):
     if busy and gui:
         # GRBM_GUI_ACTIVE is summed over the 8 XCDs, MFMA busy cycles over the 1024 SIMDs
         rep["mfma_busy_pct"] = round(100.0 * busy / (gui / 8.0 * 1024.0), 2)
+    cu_busy = raw.get("sgemm:SQ_BUSY_CU_CYCLES")
+    if busy and cu_busy:
+        # SQ_BUSY_CU_CYCLES is summed over the CUs: cycles in which a CU holds waves of the kernel
+        # (GRBM_GUI_ACTIVE also counts the dispatch overhead around a launch under the profiler)
+        rep["mfma_busy_pct_of_cu_busy"] = round(100.0 * busy / (cu_busy * 4.0), 2)
     conf, act = raw.get("sgemm:SQ_LDS_BANK_CONFLICT"), raw.get("sgemm:SQ_LDS_IDX_ACTIVE")
     if conf is not None and act:
         rep["lds_bank_conflict_pct"] = round(100.0 * conf / act, 2)
@@ -444,7 +449,7 @@ def write_counter_summary(rep, avg_ms):
                 "-d <tmp> -- python3 bench.py --inner --steps 5 --warmup 3` once per counter set)\n")
         for name, counters in PMC_PASSES.items():
             f.write(f"# pass {name}: {' '.join(counters)}\n")
-        for k in ("mfma_busy_pct", "lds_bank_conflict_pct", "fetch_scale_from_copy",
+        for k in ("mfma_busy_pct", "mfma_busy_pct_of_cu_busy", "lds_bank_conflict_pct", "fetch_scale_from_copy",
                   "write_scale_from_copy"):
             if k in rep:
                 f.write(f"{k}: {rep[k]}\n")
@@ -589,7 +594,7 @@ def main():
     }
     if counters is not None:
         line["counters"] = counters
-        for k in ("mfma_busy_pct", "lds_bank_conflict_pct"):
+        for k in ("mfma_busy_pct", "mfma_busy_pct_of_cu_busy", "lds_bank_conflict_pct"):
             if k in counters:
                 line["roofline"][k] = counters[k]
     line["dense_4096"] = bench_dense_4096(rs, args.steps, args.warmup)

@@ -566,7 +566,7 @@ struct counter_pass
     const char* counters;
 };
 const counter_pass counter_passes[] = {
-    {"mfma", "SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE SQ_INSTS_VALU_MFMA_MOPS_F32"},
+    {"mfma", "SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES GRBM_GUI_ACTIVE SQ_INSTS_VALU_MFMA_MOPS_F32"},
     {"lds", "SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE"},
     {"fetch", "FETCH_SIZE"},
     {"write", "WRITE_SIZE"},
@@ -657,7 +657,9 @@ int collect_counters(const options& opt, const char* self)
         return 2;
     }
     std::printf("\nhardware counters (rocprofv3 --pmc, mean per launch of the GEMM kernel; HBM bytes scaled by a 64 MiB copy probe)\n");
-    std::printf("%-100s %13s %20s %16s %12s\n", "Benchmark", "mfma_busy_pct", "lds_bank_conflict_pct",
+    std::printf("mfma_busy_pct: matrix-pipe busy cycles over the GPU's active cycles, which under the profiler include about\n"
+                "10 us of dispatch overhead per launch; of_cu_busy: over the cycles in which the CUs hold waves of the kernel\n");
+    std::printf("%-100s %13s %10s %20s %16s %12s\n", "Benchmark", "mfma_busy_pct", "of_cu_busy", "lds_bank_conflict_pct",
                 "hbm_MB_per_launch", "hbm_GBps");
     int failures = 0;
     for(const auto& shape : opt.shapes)
@@ -714,6 +716,11 @@ int collect_counters(const options& opt, const char* self)
                                             ? 100.0 * all["gemm:SQ_VALU_MFMA_BUSY_CYCLES"]
                                                   / (all["gemm:GRBM_GUI_ACTIVE"] / 8.0 * simds)
                                             : -1.0;
+                    // SQ_BUSY_CU_CYCLES: summed over the CUs, cycles in which a CU holds at least one wave
+                    const double busy_cu = all.count("gemm:SQ_VALU_MFMA_BUSY_CYCLES") && all["gemm:SQ_BUSY_CU_CYCLES"] > 0
+                                               ? 100.0 * all["gemm:SQ_VALU_MFMA_BUSY_CYCLES"]
+                                                     / (all["gemm:SQ_BUSY_CU_CYCLES"] * 4.0)
+                                               : -1.0;
                     const double conf = all.count("gemm:SQ_LDS_BANK_CONFLICT") && all["gemm:SQ_LDS_IDX_ACTIVE"] > 0
                                             ? 100.0 * all["gemm:SQ_LDS_BANK_CONFLICT"] / all["gemm:SQ_LDS_IDX_ACTIVE"]
                                             : -1.0;
@@ -721,7 +728,7 @@ int collect_counters(const options& opt, const char* self)
                     const double f_scale = all["copy:FETCH_SIZE"] > 0 ? probe_kib / all["copy:FETCH_SIZE"] : 1.0;
                     const double w_scale = all["copy:WRITE_SIZE"] > 0 ? probe_kib / all["copy:WRITE_SIZE"] : 1.0;
                     const double bytes = (all["gemm:FETCH_SIZE"] * f_scale + all["gemm:WRITE_SIZE"] * w_scale) * 1024.0;
-                    std::printf("%-100s %13.2f %20.2f %16.1f %12.1f\n", name.c_str(), busy, conf, bytes * 1e-6,
+                    std::printf("%-100s %13.2f %10.2f %20.2f %16.1f %12.1f\n", name.c_str(), busy, busy_cu, conf, bytes * 1e-6,
                                 avg_ms > 0 ? bytes / (avg_ms * 1e-3) * 1e-9 : -1.0);
                     std::fflush(stdout);
                 }

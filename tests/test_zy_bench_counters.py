@@ -25,10 +25,13 @@ def test_bench_float_counter_rows():
     assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
     rows = [l for l in out.stdout.splitlines() if "}/counters" in l]
     assert len(rows) == 1, out.stdout
-    m = re.search(r"\}/counters\s+(-?[\d.]+)\s+(-?[\d.]+)\s+(-?[\d.]+)\s+(-?[\d.]+)", rows[0])
+    m = re.search(r"\}/counters\s+(-?[\d.]+)\s+(-?[\d.]+)\s+(-?[\d.]+)\s+(-?[\d.]+)\s+(-?[\d.]+)", rows[0])
     assert m is not None, rows[0]
-    busy, conflicts, hbm_mb, hbm_gbps = map(float, m.groups())
+    busy, busy_of_cu, conflicts, hbm_mb, hbm_gbps = map(float, m.groups())
     assert 1.0 < busy <= 100.0
+    # over the cycles in which the CUs hold waves the figure leaves out the dispatch overhead the
+    # profiler adds around a launch, so it is the higher of the two
+    assert busy < busy_of_cu <= 100.0
     assert 0.0 <= conflicts < 5.0
     # at least the algorithmic traffic of a 1024^3 product (12.6 MB), at most a few times that
     assert 12.0 < hbm_mb < 80.0
