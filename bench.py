@@ -218,6 +218,7 @@ def bench_held_out(rs, steps, warmup):
     torch.backends.cuda.matmul.allow_tf32 = False
     names = {0: "r", 1: "c"}
     table = {key for key, _ in rs.table()}
+    table |= {(n, m, k, 1 - lb, 1 - la, 1 - lc) for (m, n, k, la, lb, lc) in table}  # mirror images: the same launch
     out = {}
     stream = torch.cuda.current_stream()
     for (m, n, k, la, lb, lc) in HELD_OUT:

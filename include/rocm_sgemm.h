@@ -230,7 +230,12 @@ int rocm_sgemm_f32_strided_batched_with_config(const rocm_sgemm_config* config,
  * nearest entry of any layout, else the built-in default.  One refinement: among the same-layout
  * entries, those of the problem's own kind (M, N and K all multiples of 4, i.e. operand
  * lines 16-byte aligned in every layout, or not) are searched first, because the two
- * kinds run different kernels (16-byte vs 4-byte direct-to-LDS loads).  Host-only, needs no GPU.
+ * kinds run different kernels (16-byte vs 4-byte direct-to-LDS loads).  A second one: the table
+ * that is searched holds, beside every tuned entry, its mirror image (N, M, K with the layouts of
+ * A and B exchanged and all three flipped, macro_m / macro_n and waves_m / waves_n exchanged)
+ * unless that problem was tuned itself: a column-major C is computed as C^T = B^T A^T, so the two
+ * are one and the same launch, and an entry tuned in one layout serves two.  rocm_sgemm_table_entry
+ * lists the tuned entries only.  Host-only, needs no GPU.
  */
 int rocm_sgemm_nearest_config(size_t M, size_t N, size_t K, int layout_a, int layout_b, int layout_c,
                               rocm_sgemm_config* out);
@@ -242,7 +247,7 @@ int rocm_sgemm_nearest_config(size_t M, size_t N, size_t K, int layout_a, int la
  * CU, reduced when it would exceed four per CU); the cost model below then prices that config,
  * those of the next three nearest entries and the larger direct-to-LDS tile shapes of the family
  * at split_k 1, 2, 3, 4, 6 and 8, and the cheapest replaces the nearest entry's config if it is
- * expected to be at least 6 % faster (distance in log size says nothing about how a tile shape
+ * expected to be at least 5 % faster (distance in log size says nothing about how a tile shape
  * divides M and N or how many tiles are left for 256 CUs).  Host-only, needs no GPU.
  */
 int rocm_sgemm_find_config(size_t M, size_t N, size_t K, int layout_a, int layout_b, int layout_c,

@@ -33,23 +33,24 @@ CUS = 256
 
 # name: (value compiled into csrc/planner.cpp, lower bound, upper bound)
 CONSTANTS = {
-    "eff_128x64": (0.992, 0.5, 1.0),   # sustained matrix-pipe efficiency by wave-tile area >= 8192
-    "eff_64x64": (0.989, 0.5, 1.0),    # >= 4096
+    "eff_128x64": (0.989, 0.5, 1.0),   # sustained matrix-pipe efficiency by wave-tile area >= 8192
+    "eff_64x64": (0.984, 0.5, 1.0),    # >= 4096
     "eff_64x32": (1.0, 0.4, 1.0),    # >= 2048
-    "eff_32x32": (0.978, 0.3, 1.0),    # smaller
-    "k_tile_64": (0.953, 0.9, 1.3),
-    "mfma_16": (0.931, 0.8, 1.1),
-    "register_staged": (1.036, 0.7, 1.1),
-    "stages_3_4": (0.957, 0.9, 1.1),
-    "masked_4_byte": (0.872, 0.6, 1.1),   # problem not all multiples of 4
-    "masked_16_byte": (0.932, 0.8, 1.05),  # ragged multiples of 4
+    "eff_32x32": (0.971, 0.3, 1.0),    # smaller
+    "k_tile_64": (0.982, 0.9, 1.3),
+    "mfma_16": (0.933, 0.8, 1.1),
+    "register_staged": (1.032, 0.7, 1.1),
+    "stages_3_4": (0.985, 0.9, 1.1),
+    "masked_4_byte": (0.861, 0.6, 1.1),   # problem not all multiples of 4
+    "masked_16_byte": (0.93, 0.8, 1.05),  # ragged multiples of 4
     "l2_tbs": (40.0, 3.0, 40.0),           # L2 -> LDS panel bandwidth over the chip
-    "l2_tbs_4_byte": (11.31, 2.0, 40.0),
-    "launch_us": (5.75, 2.0, 15.0),
-    "split_us": (2.45, 0.0, 15.0),
-    "split_tbs": (3.46, 1.0, 10.0),
-    "tail_us": (5.57, 0.0, 20.0),
-    "tail_tbs": (4.77, 1.0, 12.0),
+    "l2_tbs_4_byte": (11.75, 2.0, 40.0),
+    "launch_us": (4.44, 2.0, 15.0),
+    "split_us": (2.57, 0.0, 15.0),
+    "split_tbs": (4.15, 1.0, 10.0),
+    "tail_us": (6.15, 0.0, 20.0),
+    "tail_tbs": (5.1, 1.0, 12.0),
+    "fill_us_per_kb": (0.0281, 0.0, 0.2),  # exposed per round of tiles: the (stages - 1) K-tiles loaded before the first MFMA
 }
 NAMES = list(CONSTANTS)
 
@@ -99,15 +100,17 @@ def predict(p, c, M, N, K, batch=1):
     panels = (c["macro_m"] + c["macro_n"]) * K * 4.0 / (l2 * 1e6 / CUS)
     tile_us = (compute ** 4 + panels ** 4) ** 0.25 * per_cu
     out_mb = M * N * 4.0 / 1e6 * batch
+    # what a workgroup loads before its first MFMA: nothing overlaps it at the start of a round
+    fill_kb = (max(c["stages"], 2) - 1) * c["k_tile"] * (c["macro_m"] + c["macro_n"]) * 4.0 / 1024.0
     t = p["launch_us"]
     if c["split_k"] > 1:
         split = min(c["split_k"], k_tiles)
         groups, slots = tiles * split, CUS * per_cu
-        t += -(-groups // slots) * tile_us / split
+        t += -(-groups // slots) * (tile_us / split + p["fill_us_per_kb"] * fill_kb)
         return t + p["split_us"] + (split + 1) * out_mb / p["split_tbs"]
     tail, slots, r = tail_applies(c, tiles, k_tiles, K)
     tail = tail and batch == 1
-    t += (tiles // slots) * tile_us
+    t += (tiles // slots) * tile_us + -(-tiles // slots) * p["fill_us_per_kb"] * fill_kb
     if r > 0:
         if tail:
             tile_mb = c["macro_m"] * c["macro_n"] * 4.0 / 1e6

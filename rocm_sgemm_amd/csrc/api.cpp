@@ -182,7 +182,7 @@ int rocm_sgemm_nearest_config(size_t M, size_t N, size_t K, int layout_a, int la
     {
         return fail(ROCM_SGEMM_STATUS_INVALID_ARG, "out must be non-null and dimensions positive");
     }
-    *out = select_config(builtin_table(), builtin_table_size(), builtin_default(), M, N, K, layout_a, layout_b,
+    *out = select_config(lookup_table(), lookup_table_size(), builtin_default(), M, N, K, layout_a, layout_b,
                          layout_c);
     return ROCM_SGEMM_STATUS_OK;
 }

@@ -39,7 +39,7 @@ const rocm_sgemm_config& select_config(const tuned_entry*       table,
 /// table entry gets its entry; anything else the cheapest, by the cost model below, of the
 /// nearest entry's config (K split fitted to the problem's own tile count), those of the next
 /// three nearest entries and the larger direct-to-LDS shapes of the family at split_k 1, 2, 3, 4, 6, 8 -
-/// the nearest entry's config stays unless another is predicted at least 6 % faster.
+/// the nearest entry's config stays unless another is predicted at least 5 % faster.
 rocm_sgemm_config plan_config(size_t m, size_t n, size_t k, int layout_a, int layout_b, int layout_c,
                               size_t batch = 1);
 
@@ -55,6 +55,10 @@ bool tail_applies(const rocm_sgemm_config& config, long long tiles, long long k_
 
 const tuned_entry*       builtin_table();
 int                      builtin_table_size();
+/// The tuned table plus the mirror image (N, M, K, !b, !a, !c; tile shape exchanged) of every entry
+/// whose mirror was not tuned itself - the same launch, so the same timing; what lookups search.
+const tuned_entry*       lookup_table();
+int                      lookup_table_size();
 const rocm_sgemm_config& builtin_default();
 
 int  family_size();

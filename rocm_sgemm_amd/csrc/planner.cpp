@@ -4,6 +4,7 @@
 
 #include "dispatch.hpp"
 
+#include <algorithm>
 #include <climits>
 #include <cmath>
 #include <limits>
@@ -27,6 +28,43 @@ bool key_less(const tuned_entry& e, size_t m, size_t n, size_t k, int la, int lb
     if(e.layout_a != la) return e.layout_a < la;
     if(e.layout_b != lb) return e.layout_b < lb;
     return e.layout_c < lc;
+}
+
+// A column-major C (M x N) is computed as the row-major N x M matrix C^T = B^T * A^T with the
+// operands, the problem shape and the tile shape exchanged (run_gemm), and a row-major operand is
+// the transpose of a column-major one.  So the problem (M, N, K, a, b, c) under a config launches
+// exactly what (N, M, K, !b, !a, !c) launches under the same config with macro_m / macro_n and
+// waves_m / waves_n exchanged: an entry tuned for one is an entry for the other.
+tuned_entry mirror_of(const tuned_entry& e)
+{
+    tuned_entry r = e;
+    r.m = e.n, r.n = e.m;
+    r.layout_a = 1 - e.layout_b, r.layout_b = 1 - e.layout_a, r.layout_c = 1 - e.layout_c;
+    r.config.macro_m = e.config.macro_n, r.config.macro_n = e.config.macro_m;
+    r.config.waves_m = e.config.waves_n, r.config.waves_n = e.config.waves_m;
+    return r;
+}
+
+// The table as the library looks things up in it: every tuned entry, and the mirror image of
+// every entry whose mirror was not tuned itself; sorted by key like the tuned table.
+const std::vector<tuned_entry>& lookup_entries()
+{
+    static const std::vector<tuned_entry> entries = [] {
+        std::vector<tuned_entry> v(tuned_table, tuned_table + tuned_table_size);
+        const auto before = [](const tuned_entry& a, const tuned_entry& b) {
+            return key_less(a, b.m, b.n, b.k, b.layout_a, b.layout_b, b.layout_c);
+        };
+        for(int i = 0; i < tuned_table_size; ++i)
+        {
+            const tuned_entry m = mirror_of(tuned_table[i]);
+            // (the tuned table is sorted: binary search)
+            const tuned_entry* at = std::lower_bound(tuned_table, tuned_table + tuned_table_size, m, before);
+            if(at == tuned_table + tuned_table_size || before(m, *at)) v.push_back(m);
+        }
+        std::sort(v.begin(), v.end(), before);
+        return v;
+    }();
+    return entries;
 }
 
 // Distance between two problem sizes: sum of squared log2 ratios (the reference's measure).  The
@@ -53,9 +91,8 @@ const log_size* builtin_logs()
 {
     static const std::vector<log_size> logs = [] {
         std::vector<log_size> v;
-        v.reserve(tuned_table_size > 0 ? tuned_table_size : 1);
-        for(int i = 0; i < tuned_table_size; ++i)
-            v.push_back(logs_of(tuned_table[i].m, tuned_table[i].n, tuned_table[i].k));
+        for(const tuned_entry& e : lookup_entries())
+            v.push_back(logs_of(e.m, e.n, e.k));
         return v;
     }();
     return logs.data();
@@ -105,7 +142,7 @@ const rocm_sgemm_config& select_config(const tuned_entry*       table,
     double          best     = std::numeric_limits<double>::max();
     int             best_idx = -1;
     const log_size  here     = logs_of(m, n, k);
-    const log_size* known    = table == tuned_table ? builtin_logs() : nullptr; // else a caller's own table
+    const log_size* known    = table == lookup_entries().data() ? builtin_logs() : nullptr; // else a caller's own table
     const auto      entry_logs = [&](int i) { return known ? known[i] : logs_of(table[i].m, table[i].n, table[i].k); };
     const auto whole = [](size_t a, size_t b, size_t c) { return a % 4 == 0 && b % 4 == 0 && c % 4 == 0; };
     for(int same_kind = 1; same_kind >= 0 && best_idx < 0; --same_kind)
@@ -193,32 +230,33 @@ bool tail_applies(const rocm_sgemm_config& c, long long tiles, long long k_tiles
 // waves of one workgroup-set per CU; a tile takes the larger of its matrix-pipe time (at the
 // sustained efficiency of its wave-tile size) and the time its operand panels take from L2 into
 // LDS (small tiles are bound by that: a 64 x 64 tile needs 16 bytes per 256 flop); the stream-K tail
-// or the K split add their second pass; every launch a fixed cost.  The constants are a
+// or the K split add their second pass; every round of tiles exposes what a workgroup loads
+// before its first MFMA (stages - 1 K-tiles); every launch a fixed cost.  The constants are a
 // least-squares fit (log time, weighted towards each problem's fastest configs) to tuner sweeps of
 // the whole family over 79 problems between 192 x 192 x 8192 and 7052 x 2436 x 856, regular and
 // ragged, on MI355X (6 424 timed configs); choosing each problem's config by this model lands
-// within 4.5 % of its fastest on average (3.7 - 6.3 % on held-out thirds, worst case 30 %).  Since
-// the main loop lost its stalls the efficiencies of all wave-tile sizes are within 2 % of each
-// other.  Used to choose among candidate configs for problems that are not table entries, so
-// mainly the ordering matters.
+// within 3.9 % of its fastest on average (3.1 - 4.5 % on held-out thirds, worst case 23 %; without
+// the fill term 4.5 %, 3.7 - 6.3 % and 30 %).  Since the main loop lost its stalls the efficiencies
+// of all wave-tile sizes are within 3 % of each other.  Used to choose among candidate configs
+// for problems that are not table entries, so mainly the ordering matters.
 double predict_us(const rocm_sgemm_config& c, size_t m, size_t n, size_t k, size_t batch)
 {
     const int    waves     = c.waves_m * c.waves_n * (c.waves_k > 1 ? c.waves_k : 1);
     const int    per_cu    = waves >= 4 ? 1 : 4 / (waves < 1 ? 1 : waves);
     const double wave_area = static_cast<double>(c.macro_m / c.waves_m) * (c.macro_n / c.waves_n);
-    double       eff = wave_area >= 8192 ? 0.992 : wave_area >= 4096 ? 0.989 : wave_area >= 2048 ? 1.000 : 0.978;
-    if(c.k_tile >= 64) eff *= 0.953;
-    if(c.mfma == 16) eff *= 0.931;
-    if(c.stages == 0) eff *= 1.036;
-    if(c.stages >= 3) eff *= 0.957;
+    double       eff = wave_area >= 8192 ? 0.989 : wave_area >= 4096 ? 0.984 : wave_area >= 2048 ? 1.000 : 0.971;
+    if(c.k_tile >= 64) eff *= 0.982;
+    if(c.mfma == 16) eff *= 0.933;
+    if(c.stages == 0) eff *= 1.032;
+    if(c.stages >= 3) eff *= 0.985;
     // ragged problems run the masked kernels: 16-byte loads when every dimension is a multiple
     // of 4, 4-byte loads otherwise
     const bool aligned = m % 4 == 0 && n % 4 == 0 && k % 4 == 0;
     const bool full    = m % c.macro_m == 0 && n % c.macro_n == 0 && k % c.k_tile == 0;
     if(!aligned)
-        eff *= 0.872;
+        eff *= 0.861;
     else if(!full)
-        eff *= 0.932;
+        eff *= 0.930;
     // the products of a batch are one launch: their tiles fill the waves together
     const long long tiles   = static_cast<long long>((m + c.macro_m - 1) / c.macro_m) * ((n + c.macro_n - 1) / c.macro_n)
                               * static_cast<long long>(batch);
@@ -226,32 +264,37 @@ double predict_us(const rocm_sgemm_config& c, size_t m, size_t n, size_t k, size
     const double    kd      = static_cast<double>(k);
     const double    compute = 2.0 * c.macro_m * c.macro_n * kd / (614.5e3 * eff); // one CU's matrix pipes
     // L2 -> LDS: 40 TB/s over the CUs (the fit's upper bound: with 16-byte loads this term no longer
-    // binds any shape of the family); 11.31 TB/s for the 4-byte loads of a direct-to-LDS shape,
+    // binds any shape of the family); 11.75 TB/s for the 4-byte loads of a direct-to-LDS shape,
     // which are bound by the number of load instructions
-    const double    l2_tbs  = !aligned && c.stages != 0 ? 11.31 : 40.0;
+    const double    l2_tbs  = !aligned && c.stages != 0 ? 11.75 : 40.0;
     const double    panels  = (c.macro_m + c.macro_n) * kd * 4.0 / (l2_tbs * 1.0e6 / model_cus);
     const double    tile_us = std::sqrt(std::sqrt(compute * compute * compute * compute + panels * panels * panels * panels)) * per_cu;
     const double    out_mb  = static_cast<double>(m) * n * 4.0 / 1.0e6 * static_cast<double>(batch);
-    double          t       = 5.75; // launch, first loads, last stores
+    // what a workgroup loads before its first MFMA (stages - 1 K-tiles of both panels), in KiB:
+    // nothing overlaps it at the start of a round of tiles; 0.0281 us per KiB = 36 GB/s per CU
+    const double    fill_kb = ((c.stages > 2 ? c.stages : 2) - 1) * static_cast<double>(c.k_tile)
+                              * (c.macro_m + c.macro_n) * 4.0 / 1024.0;
+    const double    fill_us = 0.0281 * fill_kb;
+    double          t       = 4.44; // launch, last stores
     if(c.split_k > 1)
     {
         const long long split  = c.split_k < k_tiles ? c.split_k : k_tiles;
         const long long groups = tiles * split;
         const long long slots  = model_cus * per_cu;
-        t += static_cast<double>((groups + slots - 1) / slots) * tile_us / split;
-        t += 2.45 + (split + 1) * out_mb / 3.46; // second pass: launch gap, partials at ~3.5 TB/s
+        t += static_cast<double>((groups + slots - 1) / slots) * (tile_us / split + fill_us);
+        t += 2.57 + (split + 1) * out_mb / 4.15; // second pass: launch gap, partials at ~4 TB/s
         return t;
     }
     long long slots = 0, r = 0;
     const bool tail = tail_applies(c, tiles, k_tiles, k, model_cus, &slots, &r) && batch == 1;
-    t += static_cast<double>(tiles / slots) * tile_us;
+    t += static_cast<double>(tiles / slots) * tile_us + static_cast<double>((tiles + slots - 1) / slots) * fill_us;
     if(r > 0)
     {
         if(tail)
         {
             const double tile_mb = c.macro_m * c.macro_n * 4.0 / 1.0e6;
-            // second pass: launch gap, the segments at ~4.8 TB/s
-            t += tile_us * static_cast<double>(r) / slots + 5.57 + (2.0 * slots + r) * tile_mb / 4.77;
+            // second pass: launch gap, the segments at ~5 TB/s
+            t += tile_us * static_cast<double>(r) / slots + 6.15 + (2.0 * slots + r) * tile_mb / 5.10;
         }
         else
         {
@@ -302,15 +345,16 @@ namespace
 
 rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, int lc, size_t batch)
 {
-    const rocm_sgemm_config nearest
-        = select_config(tuned_table, tuned_table_size, default_config, m, n, k, la, lb, lc);
+    const tuned_entry* table      = lookup_table();
+    const int          table_size = lookup_table_size();
+    const rocm_sgemm_config nearest = select_config(table, table_size, default_config, m, n, k, la, lb, lc);
     // (the table is tuned on single products: a batch of them is planned like any other problem)
-    for(int i = 0; i < tuned_table_size && batch == 1; ++i)
+    for(int i = 0; i < table_size && batch == 1; ++i)
     {
-        const tuned_entry& e = tuned_table[i];
+        const tuned_entry& e = table[i];
         if(e.m == m && e.n == n && e.k == k && e.layout_a == la && e.layout_b == lb && e.layout_c == lc)
         {
-            return nearest; // tuned for exactly this problem
+            return nearest; // tuned for exactly this problem (or for its mirror image)
         }
     }
     // Not a table entry.  The nearest entry's config (split_k fitted to this problem) is the
@@ -321,7 +365,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     // smaller ones with waves along K, which keep a large wave tile; the 16-row tiles of 16 x 16
     // MFMAs where the problem has at most 16 rows or columns) at
     // split_k 1, 2, 3, 4, 6 and 8; the cheapest of them replaces the nearest entry's config only if
-    // the model expects it to be at least 6 % faster (the model's own error on held-out problems).
+    // the model expects it to be at least 5 % faster (above the model's error of 3 - 4.5 % on held-out problems).
     const auto aligned_kind = [](size_t a, size_t b, size_t c) { return a % 4 == 0 && b % 4 == 0 && c % 4 == 0; };
     constexpr int   max_candidates = 4;
     const log_size  here  = logs_of(m, n, k);
@@ -329,9 +373,9 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     int           idx[max_candidates];
     double        dist[max_candidates];
     int           count = 0;
-    for(int i = 0; i < tuned_table_size; ++i)
+    for(int i = 0; i < table_size; ++i)
     {
-        const tuned_entry& e = tuned_table[i];
+        const tuned_entry& e = table[i];
         if(e.layout_a != la || e.layout_b != lb || e.layout_c != lc
            || aligned_kind(e.m, e.n, e.k) != aligned_kind(m, n, k))
         {
@@ -357,7 +401,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     const double nearest_us = best_us;
     const auto   consider   = [&](const rocm_sgemm_config& c) {
         const double us = predict_us(c, m, n, k, batch);
-        if(us < best_us && us <= 0.94 * nearest_us)
+        if(us < best_us && us <= 0.95 * nearest_us)
         {
             best    = c;
             best_us = us;
@@ -365,7 +409,7 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
     };
     for(int j = 0; j < count; ++j)
     {
-        rocm_sgemm_config c = tuned_table[idx[j]].config;
+        rocm_sgemm_config c = table[idx[j]].config;
         fit_split(c, m, n, k, batch);
         consider(c);
     }
@@ -392,6 +436,16 @@ rocm_sgemm_config plan_uncached(size_t m, size_t n, size_t k, int la, int lb, in
 const tuned_entry* builtin_table()
 {
     return tuned_table;
+}
+
+const tuned_entry* lookup_table()
+{
+    return lookup_entries().data();
+}
+
+int lookup_table_size()
+{
+    return static_cast<int>(lookup_entries().size());
 }
 
 int builtin_table_size()

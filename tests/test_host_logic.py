@@ -52,6 +52,24 @@ def test_version_string():
 
 # ---- config lookup (reference generate_config.py:174-267 semantics) ----------------------------
 
+def _mirror(key, cfg):
+    """(M, N, K, a, b, c) under a config launches exactly what (N, M, K, !b, !a, !c) launches under
+    the config with macro_m / macro_n and waves_m / waves_n exchanged: a column-major C is computed
+    as C^T = B^T A^T with operands, problem and tile shape exchanged."""
+    M, N, K, a, b, c = key
+    d = cfg.as_dict()
+    d.update(macro_m=cfg.macro_n, macro_n=cfg.macro_m, waves_m=cfg.waves_n, waves_n=cfg.waves_m)
+    return (N, M, K, 1 - b, 1 - a, 1 - c), rs.Config.from_dict(d)
+
+
+def _with_mirrors(table):
+    """What the library searches: the tuned entries plus the mirror image of every entry whose
+    mirror is not a tuned entry itself, in key order."""
+    keys = {k for k, _ in table}
+    extra = [_mirror(k, cfg) for k, cfg in table]
+    return sorted(list(table) + [(k, cfg) for k, cfg in extra if k not in keys], key=lambda e: e[0])
+
+
 def _py_select(table, M, N, K, a, b, c):
     """Independent restatement of the lookup rule for cross-checking the C++ one."""
     for key, cfg in table:
@@ -88,7 +106,7 @@ def _py_plan(table, M, N, K, a, b, c):
     returned as they are; otherwise the nearest entry's config, unless one of the four nearest
     entries of the same layouts and kind (split_k fitted first) or one of the larger direct-to-LDS
     tile shapes (or smaller ones with waves along K) at split_k 1, 2, 3, 4, 6 or 8 is predicted at least
-    6 % faster."""
+    5 % faster."""
     nearest = _py_select(table, M, N, K, a, b, c).as_dict()
     if any(key == (M, N, K, a, b, c) for key, _ in table):
         return nearest
@@ -116,7 +134,7 @@ def _py_plan(table, M, N, K, a, b, c):
             candidates.append(dict(fam.as_dict(), split_k=split, group_m=4, wave_slots=0))
     for cand in candidates:
         us = rs.predict_us(cand, M, N, K)
-        if us < best_us and us <= 0.94 * nearest_us:
+        if us < best_us and us <= 0.95 * nearest_us:
             best, best_us = cand, us
     return best
 
@@ -190,11 +208,28 @@ def test_exact_hits_return_their_entry():
                                    (512, 512, 8192), (2048, 2048, 16384), (96, 4096, 4096),
                                    (1000, 1000, 4096), (5000, 5000, 5024), (640, 640, 640)])
 def test_nearest_neighbour_fallback_matches_restatement(shape):
-    table = rs.table()
+    table = _with_mirrors(rs.table())
     for a, b, c in itertools.product((0, 1), repeat=3):
         got = rs.find_config(*shape, a, b, c)
         assert got.as_dict() == _py_plan(table, *shape, a, b, c)
         assert rs.nearest_config(*shape, a, b, c).as_dict() == _py_select(table, *shape, a, b, c).as_dict()
+
+
+def test_mirror_image_of_a_tuned_entry_is_an_entry():
+    """A rectangular entry tuned in one layout serves its mirror image (transposed problem, layouts
+    of A and B exchanged and flipped, C flipped) with the tile shape exchanged - unless the mirror
+    was tuned itself, in which case its own entry wins."""
+    tuned = dict(rs.table())
+    checked = 0
+    for key, cfg in rs.table():
+        mkey, mcfg = _mirror(key, cfg)
+        assert _mirror(mkey, mcfg)[0] == key and _mirror(mkey, mcfg)[1].as_dict() == cfg.as_dict()
+        want = tuned[mkey] if mkey in tuned else mcfg
+        assert rs.find_config(*mkey).as_dict() == want.as_dict(), (key, mkey)
+        assert rs.nearest_config(*mkey).as_dict() == want.as_dict()
+        assert rs.config_supported(want, mkey[5], mkey[3], mkey[4])
+        checked += mkey not in tuned
+    assert checked > 0  # the shipped table does hold rectangular entries without a tuned mirror
 
 
 def test_whole_tile_and_ragged_problems_look_up_entries_of_their_own_kind():
@@ -236,8 +271,10 @@ def test_inherited_split_k_is_fitted_to_the_problem():
         groups = -(-m // small["macro_m"]) * -(-n // small["macro_n"]) * small["split_k"]
         inherited = -(-m // nearest["macro_m"]) * -(-n // nearest["macro_n"]) * nearest["split_k"]
         assert (small["split_k"] == 1 and small["wave_slots"] == 0) or groups >= min(128, inherited), (m, n, K, small)
-        # the plan is the nearest entry's config or one the model rates faster
-        assert small == nearest or rs.predict_us(small, m, n, K) < rs.predict_us(nearest, m, n, K)
+        # the plan is the nearest entry's config (its split fitted to this problem) or one the
+        # model rates faster than that
+        fitted = _fit_split(nearest, m, n, K)
+        assert small in (nearest, fitted) or rs.predict_us(small, m, n, K) < rs.predict_us(fitted, m, n, K)
     if tried == 0:
         pytest.skip("no row-major table entry splits K at present")
 
@@ -609,6 +646,7 @@ def test_bench_held_out_shapes_are_not_table_entries():
     assert len(bench.HELD_OUT) >= 4
     for (m, n, k, la, lb, lc) in bench.HELD_OUT:
         assert (m, n, k, la, lb, lc) not in keys
+        assert (n, m, k, 1 - lb, 1 - la, 1 - lc) not in keys  # nor its mirror image, which is the same launch
     assert len({(la, lb, lc) for (_, _, _, la, lb, lc) in bench.HELD_OUT}) >= 4  # mixed layouts
 
 
