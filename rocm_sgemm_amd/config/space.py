@@ -160,8 +160,9 @@ _BASE_SHAPES = [
     # share a CU and one's prologue and epilogue hide behind the other's main loop.  Found by the
     # tuner's exploration mode (8192 x 8192 x 1024: 1.5 % over the best shape of the family then)
     (256, 128, 16, 2, 2, 32, 2, 1),
-    # K-tiles of 64: half as many pipeline steps (barriers, waits) per unit of depth
-    (128, 128, 64, 2, 2, 32, 2, 1),
+    # K-tiles of 64: half as many pipeline steps (barriers, waits) per unit of depth (the 128 x 128
+    # form with four waves came within 1 % of the fastest shape in none of 79 sweeps and in none of
+    # 492 tuned entries; the eight-wave form above does)
     (64, 64, 64, 2, 2, 32, 2, 1),
     # waves along K: small macro tiles whose waves still own a 64 x 64 (or 64 x 32) wave tile, for
     # problems that need many tiles to fill the GPU

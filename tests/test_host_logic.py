@@ -502,12 +502,12 @@ def test_tuner_driver_finds_planted_optimum_and_merges(tmp_path):
 
 
 def test_tuner_budget_and_split_candidates():
-    run, calls = _fake_runner((128, 128, 64, 2, 2, 32, 2, 1), 4)
+    run, calls = _fake_runner((128, 128, 64, 4, 2, 32, 2, 1), 4)
     t = tune.Tuner("tuner", budget=5, runner=run, verbose=False)
     rec = t.tune_problem(1024, 1024, 16384, (0, 0, 0))
     # the family sweep is one process and always complete; the budget only stops phase 2
     assert not any(c[1] != "--sweep" for c in calls)
-    assert tuple(rec["config"][k] for k in space.SHAPE_KEYS) == (128, 128, 64, 2, 2, 32, 2, 1)
+    assert tuple(rec["config"][k] for k in space.SHAPE_KEYS) == (128, 128, 64, 4, 2, 32, 2, 1)
     assert tune.split_candidates((256, 256, 16, 2, 2, 32, 0, 1), 8192, 8192, 8192) == [1]
     assert 4 in tune.split_candidates((256, 256, 16, 2, 2, 32, 0, 1), 1024, 1024, 16384)
     assert tune.parse_layouts(["r,c,r", "col_major,row_major,col_major"]) == [(0, 1, 0), (1, 0, 1)]
