@@ -244,6 +244,27 @@ def _build(generate_config, jobs, force, tuner, verbose, LIB_PATH, OBJ_DIR, side
     return LIB_PATH
 
 
+# A tile shape from outside the shipped family whose side library the build always makes, so that
+# the exploration path (generator -> side library -> its own trial binary) is exercised end to end
+# by a GPU test without compiling anything on the GPU box: 128 x 128 x 32 with a three-stage ring.
+EXPLORE_CHECK_SHAPE = (128, 128, 32, 2, 2, 32, 3, 1)
+EXPLORE_CHECK_DIR = os.path.join(PKG_DIR, "_build", "explore_check")
+
+
+def build_explore_check(jobs=None, force=False, verbose=False):
+    """Side library + trial binary of EXPLORE_CHECK_SHAPE under EXPLORE_CHECK_DIR."""
+    sys.path.insert(0, os.path.join(PKG_DIR, "config"))
+    import space  # noqa: E402
+    if EXPLORE_CHECK_SHAPE in space.shipped_family():
+        raise RuntimeError("the exploration check's tile shape has joined the family: choose another")
+    try:
+        shapes = space.explore([EXPLORE_CHECK_SHAPE])
+        build(jobs=jobs, force=force, out_dir=EXPLORE_CHECK_DIR, shapes=shapes, verbose=verbose)
+    finally:
+        space.explore([])  # leave the family as shipped
+    return os.path.join(EXPLORE_CHECK_DIR, "config", "tuner")
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--jobs", type=int, default=None)

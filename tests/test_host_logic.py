@@ -637,6 +637,29 @@ target_link_libraries(caller PRIVATE rocm_sgemm)
     assert "rocm_sgemm4gemm" in undefined  # resolved at load time from the imported library
 
 
+def test_side_library_of_the_exploration_check_holds_the_shape_the_shipped_one_lacks():
+    """The build makes a side library with one tile shape from outside the family (a GPU test
+    times it through the side library's own trial binary).  Host part: that library's family is
+    the explored shape, its transpose and the default config's shape, and only it supports the
+    shape."""
+    from rocm_sgemm_amd import build as lib_build
+    side = os.path.join(lib_build.EXPLORE_CHECK_DIR, "librocm_sgemm.so")
+    if not os.path.exists(side):  # a tree whose build step has not run yet
+        lib_build.build_explore_check()
+    assert os.path.exists(side) and os.path.exists(os.path.join(lib_build.EXPLORE_CHECK_DIR, "config", "tuner"))
+    shape = lib_build.EXPLORE_CHECK_SHAPE
+    cfg = rs.Config.from_dict(dict(zip(space.SHAPE_KEYS, shape)))
+    assert shape not in space.shipped_family() and space.shape_ok(shape)
+    assert not rs.config_supported(cfg)
+    # in a process of its own: the loader would hand back the shipped library for the same soname
+    probe = ("import ctypes, sys; L = ctypes.CDLL(sys.argv[1]); c = (ctypes.c_int * 12)(*map(int, sys.argv[2:14])); "
+             "print(L.rocm_sgemm_config_supported(c, 0, 0, 0), L.rocm_sgemm_family_size())")
+    out = subprocess.run([sys.executable, "-c", probe, side] + [str(v) for v in cfg.as_dict().values()],
+                         capture_output=True, text=True, check=True).stdout.split()
+    default_shape = tuple(space.DEFAULT_CONFIG[k] for k in space.SHAPE_KEYS)
+    assert out == ["1", str(len({shape, space.swapped(shape), default_shape}))]
+
+
 def test_bench_held_out_shapes_are_not_table_entries():
     """bench.py's held-out rows measure the planner, so none of them may be a tuned entry."""
     sys.path.insert(0, REPO)

@@ -78,3 +78,36 @@ def test_driver_with_the_real_trial_binary_returns_a_runnable_config():
     assert entry["range"] == {"M": M, "N": N, "K": K}
     assert entry["layout"] == {"A": "row_major", "B": "col_major", "C": "row_major"}
     assert set(entry["config"]) == set(space.CONFIG_KEYS)
+
+
+def test_exploration_times_a_tile_shape_from_outside_the_family():
+    """tune.py --explore end to end on the GPU: the family sweep on the shipped trial binary, then
+    a tile shape the library does not ship (128 x 128 x 32 with a three-stage ring), compiled by
+    the build into a side library with a trial binary of its own, timed and verified there
+    (a trial whose result is wrong says `ok 0` and is dropped, so a record means `ok 1`)."""
+    from rocm_sgemm_amd import build as lib_build
+    shape = lib_build.EXPLORE_CHECK_SHAPE
+    side_tuner = os.path.join(lib_build.EXPLORE_CHECK_DIR, "config", "tuner")
+    assert os.path.exists(side_tuner), "the build makes the side library (build_explore_check)"
+    assert shape not in space.shipped_family() and not rs.config_supported(dict(zip(space.SHAPE_KEYS, shape)))
+    print("CASE tuner explore", shape, flush=True)
+    fam = tune.Tuner(TUNER, budget=5, iters=3, verbose=False)
+    try:
+        found = tune.explore([(1024, 768, 2048)], [(0, 0, 0)], [shape], fam, lib_build.EXPLORE_CHECK_DIR,
+                             side_build=lambda out_dir, shapes: side_tuner, log=lambda *a: None)
+    finally:
+        space.explore([])  # leave the family as shipped for the other tests
+    assert len(found) == 1
+    rec = found[0]
+    assert rec["family"] is not None and rec["family"]["avg_ms"] > 0
+    assert tuple(rec["family"]["config"][k] for k in space.SHAPE_KEYS) in space.shipped_family()
+    assert rec["explored"] is not None, "the explored shape produced no verified trial"
+    got = tuple(rec["explored"]["config"][k] for k in space.SHAPE_KEYS)
+    assert got in (shape, space.swapped(shape)) and rec["explored"]["avg_ms"] > 0
+    # both were timed on the same problem: the two figures are of one order
+    assert 0.2 < rec["explored"]["avg_ms"] / rec["family"]["avg_ms"] < 5.0
+    # the shipped library refuses the shape, the side library's trial binary runs it
+    cfg = dict(zip(space.SHAPE_KEYS, shape), split_k=1, group_m=4, wave_slots=0, partial_sums=0)
+    argv = ["1024", "768", "2048"] + [str(cfg[k]) for k in space.CONFIG_KEYS] + ["0", "0", "0", "3"]
+    assert subprocess.run([TUNER] + argv, capture_output=True, text=True, timeout=120).returncode == 3
+    assert subprocess.run([side_tuner] + argv, capture_output=True, text=True, timeout=120).returncode == 0
