@@ -263,6 +263,52 @@ def test_linearity_in_power_of_two_scale_is_exact():
     assert torch.equal(_run_device(dA, dB * 0.25, M, N, K, 0, 1, 0), base * 0.25)
 
 
+def test_subnormal_inputs_and_results_are_not_flushed():
+    """The reference multiplies with ordinary fp32 FMAs, which on its targets keep subnormal values
+    (gradual underflow), and its CPU check does the same.  The matrix-core path must not flush
+    them: products and sums in the subnormal range (around 4e-39, below the smallest normal
+    1.18e-38) and subnormal inputs (around 1e-40) come out as the fp64 product says, to the
+    precision subnormal numbers have (their spacing is 1.4e-45, i.e. about 4e-7 of these sums per
+    rounding), in a full-tile, a ragged and a column-major case and through a K split."""
+    rng = np.random.default_rng(3)
+    for (M, N, K, la, lb, lc, split) in [(64, 64, 64, 0, 0, 0, 1), (300, 260, 100, 0, 1, 0, 1),
+                                         (512, 256, 96, 1, 0, 1, 1), (128, 128, 512, 0, 0, 0, 4)]:
+        _announce("subnormal", M, N, K, la, lb, lc, split)
+        cfg = dict(rs.find_config(M, N, K, la, lb, lc).as_dict(), split_k=split)
+        for scale_a, scale_b in ((1e-25, 1e-15), (1e-40, 1e10)):
+            A = (rng.uniform(0.5, 1.0, (M, K)) * scale_a).astype(np.float32)
+            B = (rng.uniform(0.5, 1.0, (K, N)) * scale_b).astype(np.float32)
+            assert scale_a > 1e-30 or float(A.max()) < 1.2e-38  # the second case feeds subnormal inputs
+            want = A.astype(np.float64) @ B.astype(np.float64)
+            got = run_gemm(oracle.to_storage(A, la), oracle.to_storage(B, lb), M, N, K, la, lb, lc, config=cfg)
+            got = got.reshape(M, N) if lc == 0 else got.reshape(N, M).T
+            assert not (got == 0).any(), (M, N, K, scale_a)
+            assert float(np.max(np.abs(got - want) / want)) < 4e-7 * K, (M, N, K, scale_a)
+
+
+def test_nan_and_infinity_propagate_as_ieee_says_and_nowhere_else():
+    """A NaN in row i of A makes row i of C NaN, an infinity (with positive B) makes its row
+    infinite, and every other row equals, bit for bit, what it is without them - in a ragged problem
+    (masked kernels), a full-tile one and through a K split, for both storage orders of C."""
+    rng = np.random.default_rng(8)
+    for (M, N, K, la, lb, lc, split) in [(300, 260, 100, 0, 0, 0, 1), (256, 256, 128, 1, 1, 1, 1),
+                                         (255, 257, 1029, 0, 1, 0, 3)]:
+        _announce("nan_inf", M, N, K, la, lb, lc, split)
+        cfg = dict(rs.find_config(M, N, K, la, lb, lc).as_dict(), split_k=split)
+        A = rng.uniform(-1.0, 1.0, (M, K)).astype(np.float32)
+        B = rng.uniform(0.5, 1.0, (K, N)).astype(np.float32)
+        def product(a):
+            flat = run_gemm(oracle.to_storage(a, la), oracle.to_storage(B, lb), M, N, K, la, lb, lc, config=cfg)
+            return flat.reshape(M, N) if lc == 0 else flat.reshape(N, M).T
+        clean = product(A)
+        special = A.copy()
+        special[5, 7], special[9, K - 1], special[M - 1, 0] = np.nan, np.inf, -np.inf
+        got = product(special)
+        assert np.isnan(got[5]).all() and (got[9] == np.inf).all() and (got[M - 1] == -np.inf).all()
+        others = [i for i in range(M) if i not in (5, 9, M - 1)]
+        assert np.array_equal(got[others].view(np.uint32), clean[others].view(np.uint32))
+
+
 def test_run_to_run_determinism_including_split_k():
     import torch
     M, N, K = 512, 384, 4096
