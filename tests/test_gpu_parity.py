@@ -950,6 +950,34 @@ def test_matches_the_reference_gpu_kernel(size, la, lb, lc):
             assert err <= REL_TOL, err
 
 
+# ---- every tuned entry, at its own size ------------------------------------------------------------------
+
+def test_every_table_entry_is_exact_on_integers_at_its_own_size():
+    """Each of the table's (M, N, K, layouts) problems through the default dispatcher, i.e. under
+    the config tuned for it (tile shape, K split, stream-K tail, band height), on integer-valued
+    inputs: bit-exact against the fp64 product.  The tuner's own gate is a sampled check at
+    tuning time; this one is complete and runs on the table as shipped."""
+    import torch
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(11)
+    stream = torch.cuda.current_stream()
+    table = rs.table()
+    assert len(table) > 300
+    for (M, N, K, la, lb, lc), cfg in table:
+        _announce("table_entry", M, N, K, la, lb, lc)
+        A = torch.randint(-4, 5, (M, K), generator=g, device="cuda:0").float()
+        B = torch.randint(-4, 5, (K, N), generator=g, device="cuda:0").float()
+        dA = (A if la == 0 else A.t().contiguous()).reshape(-1)
+        dB = (B if lb == 0 else B.t().contiguous()).reshape(-1)
+        dC = torch.full((M * N,), float("nan"), device="cuda:0")
+        rs.gemm(dC, dA, dB, M, N, K, lc, la, lb, stream=stream)
+        want = (A.double() @ B.double()).float()
+        want = (want if lc == 0 else want.t().contiguous()).reshape(-1)
+        torch.cuda.synchronize()
+        assert torch.equal(dC, want), (M, N, K, la, lb, lc, cfg)
+        del A, B, dA, dB, dC, want
+
+
 # ---- randomised sweep through the default dispatcher ---------------------------------------------------
 
 def test_random_problems_exact_on_integers():
