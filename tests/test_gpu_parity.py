@@ -953,8 +953,8 @@ def test_matches_the_reference_gpu_kernel(size, la, lb, lc):
 # ---- every tuned entry, at its own size ------------------------------------------------------------------
 
 def test_every_table_entry_is_exact_on_integers_at_its_own_size():
-    """Each of the table's (M, N, K, layouts) problems through the default dispatcher, i.e. under
-    the config tuned for it (tile shape, K split, stream-K tail, band height), on integer-valued
+    """Each of the table's (M, N, K, layouts) problems, and its mirror image, through the default
+    dispatcher, i.e. under the config tuned for it (tile shape, K split, stream-K tail, band height), on integer-valued
     inputs: bit-exact against the fp64 product.  The tuner's own gate is a sampled check at
     tuning time; this one is complete and runs on the table as shipped."""
     import torch
@@ -963,7 +963,13 @@ def test_every_table_entry_is_exact_on_integers_at_its_own_size():
     stream = torch.cuda.current_stream()
     table = rs.table()
     assert len(table) > 300
-    for (M, N, K, la, lb, lc), cfg in table:
+    # and the mirror image of every entry (N, M, K, layouts of A and B exchanged, all three flipped),
+    # which the lookup serves with the entry's config, tile shape exchanged
+    keys = {key for key, _ in table}
+    problems = sorted(keys | {(N, M, K, 1 - lb, 1 - la, 1 - lc) for (M, N, K, la, lb, lc) in keys})
+    assert len(problems) > len(keys)
+    for (M, N, K, la, lb, lc) in problems:
+        cfg = rs.find_config(M, N, K, la, lb, lc)
         _announce("table_entry", M, N, K, la, lb, lc)
         A = torch.randint(-4, 5, (M, K), generator=g, device="cuda:0").float()
         B = torch.randint(-4, 5, (K, N), generator=g, device="cuda:0").float()
