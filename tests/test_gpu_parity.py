@@ -984,6 +984,43 @@ def test_every_table_entry_is_exact_on_integers_at_its_own_size():
         del A, B, dA, dB, dC, want
 
 
+def test_random_mid_and_large_problems_exact_on_integers():
+    """600 seeded random problems of the sizes the planner is for (64 ... 6000 per dimension, a third
+    multiples of 64, a third multiples of 4, a third arbitrary; all layouts), none of them a table
+    entry, so each runs whatever the planner chooses - an inherited or fitted K split, a stream-K
+    tail, a tile shape from the cost model: bit-exact against the fp64 product."""
+    import random
+    import torch
+    rnd = random.Random(2024)
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(12)
+    stream = torch.cuda.current_stream()
+    keys = {key for key, _ in rs.table()}
+    kinds = set()
+    done = 0
+    while done < 600:
+        step = rnd.choice([64, 4, 1])
+        M, N, K = (max(step, int(2 ** rnd.uniform(6, 12.55)) // step * step) for _ in range(3))
+        la, lb, lc = (rnd.randint(0, 1) for _ in range(3))
+        if 2.0 * M * N * K > 2.0 * 4096 ** 3 or (M, N, K, la, lb, lc) in keys:
+            continue
+        done += 1
+        cfg = rs.find_config(M, N, K, la, lb, lc)
+        kinds.add(("split" if cfg.split_k > 1 else "plain", cfg.waves_k > 1, cfg.stages))
+        _announce("random_large", M, N, K, la, lb, lc, cfg)
+        A = torch.randint(-4, 5, (M, K), generator=g, device="cuda:0").float()
+        B = torch.randint(-4, 5, (K, N), generator=g, device="cuda:0").float()
+        dA = (A if la == 0 else A.t().contiguous()).reshape(-1)
+        dB = (B if lb == 0 else B.t().contiguous()).reshape(-1)
+        dC = torch.full((M * N,), float("nan"), device="cuda:0")
+        rs.gemm(dC, dA, dB, M, N, K, lc, la, lb, stream=stream)
+        want = (A.double() @ B.double()).float()
+        want = (want if lc == 0 else want.t().contiguous()).reshape(-1)
+        torch.cuda.synchronize()
+        assert torch.equal(dC, want), (M, N, K, la, lb, lc, cfg)
+    assert len(kinds) >= 4  # the draw exercises K splits, waves along K and several ring depths
+
+
 # ---- randomised sweep through the default dispatcher ---------------------------------------------------
 
 def test_random_problems_exact_on_integers():
