@@ -227,8 +227,8 @@ int main(int argc, char** argv)
             rc |= run_case<tile_config<64, 32, 64, 1, 1, 32, true, false, false, 3, 4, 4, 4>>(
                 "64x32x64, 4 waves along K, 3 stages", 128, 4096, 4096, 4, 1);
         else if(c == "ragged")
-            rc |= run_case<tile_config<64, 64, 32, 2, 2, 32, true, false, true, 2, 1, 1, 1>>(
-                "64x64x32, 2x2 waves, 2 stages, masked with 4-byte loads", 1000, 3000, 777, 16, 1);
+            rc |= run_case<tile_config<64, 64, 32, 2, 2, 32, true, false, true, 3, 1, 1, 1>>(
+                "64x64x32, 2x2 waves, 3 stages, masked with 4-byte loads", 1000, 3000, 777, 4, 1);
         else if(c == "deepk")
             rc |= run_case<tile_config<64, 64, 128, 1, 1, 32, true, false, false, 2, 4, 4, 4>>(
                 "64x64x128, 4 waves along K, 2 stages", 1024, 1024, 16384, 4, 1);

@@ -153,6 +153,11 @@ _BASE_SHAPES = [
     (128, 128, 32, 2, 2, 32, 2, 1),
     (128, 64, 32, 2, 2, 32, 3, 1),
     (64, 64, 32, 2, 2, 32, 2, 1),
+    # the same tile with a three-stage ring, for problems whose operand lines are not 16-byte
+    # aligned: their 4-byte loads take longer to land, and a K-tile more in flight covers that
+    # (1000 x 3000 x 777: 2 - 3 % in the six layouts with such loads on the deep side, 3001 x 1001 x
+    # 1501 2.7 %; aligned problems and 1023^3 are 0.5 - 2 % better off with two stages)
+    (64, 64, 32, 2, 2, 32, 3, 1),
     # eight waves: two per SIMD cover each other's stalls in prologue and epilogue
     (256, 128, 32, 4, 2, 32, 2, 1),
     (128, 128, 64, 4, 2, 32, 2, 1),
