@@ -11,7 +11,8 @@ Input: logs of `tuner --sweep M N K a b c --splits 1,2,4,8 --groups 4` (one line
 every problem of fit_problems.txt, the list the compiled constants were fitted on.  The fit minimises the squared error of log(time), weighting each config
 by exp(-(t / t_best - 1) / 0.25) so that the ordering among a problem's fast configs matters most.
 
-usage: fit_cost_model.py --collect DIR [--iters n]     sweeps the problems of fit_problems.txt into DIR
+usage: fit_cost_model.py --collect DIR [--iters n] [--first i] [--count n]
+                                                        sweeps the problems (all, or n from the i-th) of fit_problems.txt into DIR
        fit_cost_model.py 'DIR/sweep_*.log' [...]       prints the fitted constants, the quality of
                                                         picking configs by the model (chosen / best
                                                         time per problem) and a 3-fold check
@@ -180,14 +181,15 @@ def fit(data):
     return dict(zip(NAMES, least_squares(residuals, x0, bounds=(lo, hi)).x))
 
 
-def collect(out_dir, iters=20):
-    """Sweeps every problem of fit_problems.txt with the tuner binary (needs a GPU)."""
+def collect(out_dir, iters=20, first=0, count=None):
+    """Sweeps the problems [first, first + count) of fit_problems.txt with the tuner binary (needs a GPU)."""
     import os
     import subprocess
     here = os.path.dirname(os.path.abspath(__file__))
     os.makedirs(out_dir, exist_ok=True)
     with open(os.path.join(here, "fit_problems.txt")) as f:
         problems = [tuple(map(int, line.split())) for line in f if line.strip() and not line.startswith("#")]
+    problems = problems[first:first + count if count is not None else None]
     for i, (M, N, K) in enumerate(problems):
         log = os.path.join(out_dir, f"sweep_{M}_{N}_{K}.log")
         cmd = [os.path.join(here, "tuner"), "--sweep", str(M), str(N), str(K), "0", "0", "0", "--iters",
@@ -205,8 +207,8 @@ def main(argv):
         print(__doc__)
         return 2
     if argv[1] == "--collect":
-        iters = int(argv[argv.index("--iters") + 1]) if "--iters" in argv else 20
-        return collect(argv[2], iters)
+        opt = lambda name, default: int(argv[argv.index(name) + 1]) if name in argv else default  # noqa: E731
+        return collect(argv[2], opt("--iters", 20), opt("--first", 0), opt("--count", None))
     data = load(argv[1:])
     if not data:
         print("no sweep logs matched", file=sys.stderr)
